@@ -1,0 +1,164 @@
+"""CPU restatement of the reference's eager workloads (the numerical definition of the hot path).
+
+TEST INFRASTRUCTURE (see `oracle/__init__.py`): the checker for the HIP kernels and the CPU baseline
+that `bench.py` times.  Never imported by the product package.
+
+Same torch ops, same order, same dtype at every step as the reference, so the rounding points are
+the reference's: QK^T rounded to fp16, divided by sqrt(D) in fp16, fp16 mask added, softmax in fp32,
+P rounded to fp16 before PV.
+
+How each function is pinned (tests/test_oracle_pins.py, tests/test_oracle_golden.py):
+  attn_forward       torch's F.scaled_dot_product_attention(is_causal=True) in fp32; row 0 == v[0]
+                     bit-exact; q == 0 -> prefix means of V; fp64 brute force for S <= 64.
+  h2o_forward        sum_j score_j == Sq; q == 0 -> score_j = H_S - H_j (harmonic numbers);
+                     score_{S-1} == p_{S-1,S-1}; fp64 brute force.
+  roco_forward       sums as h2o; q == 0 -> sumsq_j = sum_{i>=j} (i+1)^-2; 0 <= sumsq <= sum.
+  keyformer_forward  exp_rand == 1, tau == 1 -> kf_score == h2o score; tau -> inf -> uniform closed
+                     form; sum_j == Sq; fp64 brute force with random noise.
+  ea_forward         V == c -> O == c; Q == K == 0 -> O = mean_s V; fp64 brute force.
+  sima_forward       sum_s |Qhat| == 1; scale invariance in Q and K; fp64 brute force.
+The reference holds no golden vectors or tests for this path, so none can be checked against; no
+function of this file is "parity unpinned".
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _masked_scores_probs(q, k):
+  """Shared prefix of every softmax case (cases/kernels/h2o.py:19-31, identical in attn.py:19-31,
+  kf.py:20-32, roco.py:19-37).  q,k: [B,S,H,D].  Returns (scores fp16 masked [B,H,Sq,Skv], probs fp32)."""
+  q_len, kv_len = q.shape[1], k.shape[1]
+  head_dim = q.shape[3]
+  mask = torch.full((1, 1, q_len, kv_len), -torch.inf, device=q.device, dtype=q.dtype)
+  mask = torch.triu(mask, diagonal=kv_len - q_len + 1)
+  qt = q.transpose(1, 2)
+  kt = k.transpose(1, 2)
+  scores = torch.matmul(qt, kt.transpose(-2, -1)) / math.sqrt(head_dim)
+  scores += mask
+  probs = F.softmax(scores.float(), dim=-1)
+  return scores, probs
+
+
+def _out(probs, q, v):
+  """cases/kernels/h2o.py:32,38: P rounded to the input dtype, PV, back to [B,Sq,H,D]."""
+  B, q_len, H, D = q.shape
+  out = torch.matmul(probs.to(q.dtype), v.transpose(1, 2)).transpose(1, 2).contiguous()
+  return out.view(B, q_len, H, D)
+
+
+def attn_forward(q, k, v):
+  """Causal softmax attention, cases/kernels/attn.py:18-34.  q,k,v [B,S,H,D] -> out [B,Sq,H,D]."""
+  _, probs = _masked_scores_probs(q, k)
+  return _out(probs, q, v)
+
+
+def h2o_forward(q, k, v):
+  """H2O, cases/kernels/h2o.py:18-38: attention + per-key accumulated probability
+  h2o_score[b,h,j] = sum_i probs[b,h,i,j] (fp32, [B,H,Skv])."""
+  _, probs = _masked_scores_probs(q, k)
+  out = _out(probs, q, v)
+  h2o_score = probs.sum(dim=2)
+  return out, h2o_score.view(q.shape[0], q.shape[2], k.shape[1])
+
+
+def roco_forward(q, k, v):
+  """RoCo, cases/kernels/roco.py:18-48 (group_size == 1 branch, asserted at :16): attention + per-key
+  sum and sum of squares of the probabilities over query rows (both fp32 [B,H,Skv])."""
+  _, probs = _masked_scores_probs(q, k)
+  out = _out(probs, q, v)
+  roco_score = probs.sum(dim=2)
+  roco_sq_score = (probs ** 2).sum(dim=2)
+  shp = (q.shape[0], q.shape[2], k.shape[1])
+  return out, roco_score.view(shp), roco_sq_score.view(shp)
+
+
+def keyformer_forward(q, k, v, exp_rand, tau=1.5):
+  """KeyFormer, cases/kernels/kf.py:19-42 (tau default :8): attention (unperturbed O) + per-key column
+  sum of softmax((masked fp16 scores as fp32 + gumbels) / tau) with gumbels = -log(exp_rand)."""
+  scores, probs = _masked_scores_probs(q, k)
+  out = _out(probs, q, v)
+  gumbels = -exp_rand.log()
+  kf_score = (scores.float() + gumbels) / tau
+  kf_score = F.softmax(kf_score.float(), dim=-1)
+  kf_score = kf_score.sum(dim=2)
+  return out, kf_score.view(q.shape[0], q.shape[2], k.shape[1])
+
+
+def ea_forward(q, k, v):
+  """EA linear-attention core, bench/ea.mlir:13-17 with softmax = exp/sum over `dim`
+  (lib/Dialect/Asuka/Transforms/LowerComplexReduce.cpp:21-41): Qs = softmax(Q, dim=D),
+  Ks = softmax(K, dim=S), KV = Ks^T V, O = Qs KV.  q,k,v [B,S,H,D] fp16; the reference graph is f32, so
+  the internal math is fp32 and O is rounded once to the input dtype."""
+  qf, kf, vf = (t.transpose(1, 2).float() for t in (q, k, v))  # [B,H,S,D]
+  qs = F.softmax(qf, dim=3)
+  ks = F.softmax(kf, dim=2)
+  kv = torch.matmul(ks.transpose(-2, -1), vf)  # [B,H,D,D]
+  out = torch.matmul(qs, kv)
+  return out.transpose(1, 2).contiguous().to(q.dtype)
+
+
+def sima_forward(q, k, v, normalize_q=True, out_dtype=None):
+  """SimA linear-attention core, bench/sima.mlir:13-17 with normalize(Lp=1) = x / sum(|x|) over `dim`,
+  keep-dim, signed numerator (LowerComplexReduce.cpp:43-69): Qh = Q/sum_s|Q|, Kh = K/sum_s|K| per
+  (b,h,channel), O = Qh (Kh^T V).  normalize_q=False reproduces the .mlir's use of the raw Q at :17."""
+  qf, kf, vf = (t.transpose(1, 2).float() for t in (q, k, v))
+  kh = kf / kf.abs().sum(dim=2, keepdim=True)
+  qh = qf / qf.abs().sum(dim=2, keepdim=True) if normalize_q else qf
+  kv = torch.matmul(kh.transpose(-2, -1), vf)
+  out = torch.matmul(qh, kv)
+  return out.transpose(1, 2).contiguous().to(out_dtype or q.dtype)
+
+
+# ---------------------------------------------------------------------------------------------------
+# Input recipes and epilogues
+
+
+def prepare_inputs(B, S, H, D, seed=0, dtype=torch.float16, kv_len=None):
+  """Input recipe of every case's prepare() (cases/kernels/attn.py:36-39): q, k, v ~ N(0,1) drawn in
+  that order in the target dtype, here from the seeded CPU generator (cases/attn.py:89)."""
+  g = torch.Generator(device="cpu")
+  g.manual_seed(seed)
+  kv_len = S if kv_len is None else kv_len
+  q = torch.randn(B, S, H, D, dtype=dtype, generator=g)
+  k = torch.randn(B, kv_len, H, D, dtype=dtype, generator=g)
+  v = torch.randn(B, kv_len, H, D, dtype=dtype, generator=g)
+  return q, k, v
+
+
+def prepare_exp_rand(B, H, Sq, Skv, seed=0):
+  """Noise recipe of KeyFormer.prepare (cases/kernels/kf.py:48): 1 + |N(0,1)|, fp32."""
+  g = torch.Generator(device="cpu")
+  g.manual_seed(seed + 7919)
+  return 1 + torch.randn(B, H, Sq, Skv, dtype=torch.float32, generator=g).abs()
+
+
+def heavy_hitters(score, k):
+  """Top-k key indices per head of a [B,H,S] score, descending by score.  Not in the reference (its
+  H2O case stops at the score, cases/kernels/h2o.py:34-38); the measured configuration asks for k=S/8."""
+  return torch.topk(score, k, dim=-1, largest=True, sorted=True).indices
+
+
+def roco_mean_var(roco_score, roco_sq_score, q_len):
+  """Mean and (population) variance over the q_len query rows from RoCo's sum and sum of squares."""
+  mean = roco_score / q_len
+  return mean, roco_sq_score / q_len - mean * mean
+
+
+def chunked_over_heads(fn, tensors, head_chunk, extra=(), **kw):
+  """Evaluate fn on slices of the head axis (dim 2 of q/k/v; dim 1 of [B,H,...] extras and results) and
+  concatenate: heads are independent, so results are identical while peak memory is bounded."""
+  H = tensors[0].shape[2]
+  pieces = []
+  for h0 in range(0, H, head_chunk):
+    sl = slice(h0, min(H, h0 + head_chunk))
+    args = [t[:, :, sl].contiguous() for t in tensors] + [e[:, sl] for e in extra]
+    res = fn(*args, **kw)
+    pieces.append(res if isinstance(res, tuple) else (res,))
+  outs = []
+  for idx in range(len(pieces[0])):
+    parts = [p[idx] for p in pieces]
+    # O is [B,S,H,D] (head axis 2); scores are [B,H,S] (head axis 1)
+    outs.append(torch.cat(parts, dim=2 if parts[0].dim() == 4 else 1))
+  return outs[0] if len(outs) == 1 else tuple(outs)

@@ -1,0 +1,62 @@
+"""Independent fp64 definitions of the workloads, written from the mathematics (explicit loops over
+batch and head, numpy float64, no shared code with `oracle/`), used only to pin the oracle on tiny
+shapes: a dropped term, wrong sign, wrong axis or off-by-one mask in the oracle fails against these."""
+import numpy as np
+
+
+def _probs(q, k, b, h):
+  Sq, Skv, D = q.shape[1], k.shape[1], q.shape[3]
+  s = q[b, :, h, :].astype(np.float64) @ k[b, :, h, :].astype(np.float64).T / np.sqrt(D)
+  for i in range(Sq):
+    for j in range(Skv):
+      if j > i + (Skv - Sq):
+        s[i, j] = -np.inf
+  e = np.exp(s - s.max(axis=1, keepdims=True))
+  return s, e / e.sum(axis=1, keepdims=True)
+
+
+def attention_stats(q, k, v, exp_rand=None, tau=1.0):
+  """Returns O [B,Sq,H,D], colsum [B,H,Skv], colsumsq [B,H,Skv], kf [B,H,Skv] (None without noise)."""
+  q, k, v = (t.numpy() if hasattr(t, "numpy") else t for t in (q, k, v))
+  B, Sq, H, D = q.shape
+  Skv = k.shape[1]
+  O = np.zeros((B, Sq, H, D)); cs = np.zeros((B, H, Skv)); cq = np.zeros((B, H, Skv))
+  kf = None if exp_rand is None else np.zeros((B, H, Skv))
+  for b in range(B):
+    for h in range(H):
+      s, p = _probs(q, k, b, h)
+      O[b, :, h, :] = p @ v[b, :, h, :].astype(np.float64)
+      cs[b, h] = p.sum(axis=0)
+      cq[b, h] = (p * p).sum(axis=0)
+      if exp_rand is not None:
+        e = exp_rand[b, h].numpy().astype(np.float64) if hasattr(exp_rand, "numpy") else exp_rand[b, h]
+        z = (s - np.log(e)) / tau
+        w = np.exp(z - z.max(axis=1, keepdims=True))
+        kf[b, h] = (w / w.sum(axis=1, keepdims=True)).sum(axis=0)
+  return O, cs, cq, kf
+
+
+def ea(q, k, v):
+  q, k, v = (t.numpy().astype(np.float64) for t in (q, k, v))
+  B, S, H, D = q.shape
+  O = np.zeros((B, S, H, D))
+  for b in range(B):
+    for h in range(H):
+      Q, K, V = q[b, :, h], k[b, :, h], v[b, :, h]
+      qs = np.exp(Q) / np.exp(Q).sum(axis=1, keepdims=True)      # over channels
+      ks = np.exp(K) / np.exp(K).sum(axis=0, keepdims=True)      # over tokens
+      O[b, :, h] = qs @ (ks.T @ V)
+  return O
+
+
+def sima(q, k, v, normalize_q=True):
+  q, k, v = (t.numpy().astype(np.float64) for t in (q, k, v))
+  B, S, H, D = q.shape
+  O = np.zeros((B, S, H, D))
+  for b in range(B):
+    for h in range(H):
+      Q, K, V = q[b, :, h], k[b, :, h], v[b, :, h]
+      kh = K / np.abs(K).sum(axis=0, keepdims=True)
+      qh = Q / np.abs(Q).sum(axis=0, keepdims=True) if normalize_q else Q
+      O[b, :, h] = qh @ (kh.T @ V)
+  return O

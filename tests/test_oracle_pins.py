@@ -1,0 +1,246 @@
+"""Pins the CPU oracle: library routine, closed forms, invariants and fp64 brute force (CPU only).
+
+The reference has no tests, fixtures or golden vectors for this path, so the oracle is pinned by what
+the mathematics fixes.  Each check is chosen so that a plausible mistake (mask off by one, wrong softmax
+axis, sum over the wrong dimension, dropped 1/tau, sign of the Gumbel term, transposed K^T V) fails it.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from tests import brute
+
+
+def _inputs(B=1, S=64, H=2, D=64, seed=0, kv_len=None):
+  return oracle.prepare_inputs(B, S, H, D, seed=seed, kv_len=kv_len)
+
+
+# ------------------------------------------------------------------ attention output
+
+@pytest.mark.parametrize("S,D", [(64, 64), (128, 128), (96, 128)])
+def test_attn_matches_sdpa_fp32(S, D):
+  q, k, v = _inputs(S=S, D=D)
+  out = oracle.attn_forward(q, k, v)
+  ref = F.scaled_dot_product_attention(q.transpose(1, 2).float(), k.transpose(1, 2).float(),
+                                       v.transpose(1, 2).float(), is_causal=True).transpose(1, 2)
+  assert out.dtype == torch.float16 and out.shape == q.shape
+  assert (out.float() - ref).abs().max() < 4e-3  # fp16 rounding points of the eager definition
+
+
+def test_attn_row0_is_v0_bit_exact():
+  q, k, v = _inputs(S=128, D=128)
+  out = oracle.attn_forward(q, k, v)
+  assert torch.equal(out[:, 0], v[:, 0])
+
+
+def test_attn_zero_q_gives_prefix_means():
+  q, k, v = _inputs(S=64, D=64)
+  out = oracle.attn_forward(torch.zeros_like(q), k, v)
+  ref = v.float().cumsum(dim=1) / torch.arange(1, 65).view(1, -1, 1, 1)
+  assert (out.float() - ref).abs().max() < 2e-3
+
+
+def test_attn_rectangular_mask_offset():
+  # Sq < Skv: row i sees keys j <= i + (Skv - Sq) (triu diagonal = Skv - Sq + 1)
+  q, k, v = _inputs(S=32, D=64, kv_len=80)
+  out = oracle.attn_forward(q, k, v)
+  O, _, _, _ = brute.attention_stats(q, k, v)
+  assert np.abs(out.float().numpy() - O).max() < 4e-3
+
+
+# ------------------------------------------------------------------ column statistics
+
+def test_h2o_brute_force_and_invariants():
+  q, k, v = _inputs(B=2, S=64, H=2, D=64, seed=3)
+  out, score = oracle.h2o_forward(q, k, v)
+  O, cs, _, _ = brute.attention_stats(q, k, v)
+  assert score.dtype == torch.float32 and score.shape == (2, 2, 64)
+  assert np.abs(out.float().numpy() - O).max() < 4e-3
+  assert np.abs(score.numpy() - cs).max() / np.abs(cs).max() < 2e-3
+  # rows of P sum to one => total mass is Sq per (b,h)
+  assert torch.allclose(score.sum(-1), torch.full((2, 2), 64.0), rtol=1e-5)
+  # the last key is seen by the last query only: score_{S-1} = p_{S-1,S-1}
+  scores, probs = oracle.cases._masked_scores_probs(q, k)
+  assert torch.equal(score[..., -1], probs[..., -1, -1])
+
+
+def test_h2o_zero_q_harmonic_closed_form():
+  S = 96
+  q, k, v = _inputs(S=S, D=64)
+  _, score = oracle.h2o_forward(torch.zeros_like(q), k, v)
+  # uniform causal probs: p_ij = 1/(i+1) for j <= i  =>  score_j = sum_{i>=j} 1/(i+1) = H_S - H_j
+  harm = np.concatenate([[0.0], np.cumsum(1.0 / np.arange(1, S + 1))])
+  ref = harm[S] - harm[:S]
+  assert np.abs(score[0, 0].numpy() - ref).max() < 1e-5
+
+
+def test_roco_closed_form_and_bounds():
+  S = 80
+  q, k, v = _inputs(S=S, D=64, seed=1)
+  _, s1, s2 = oracle.roco_forward(torch.zeros_like(q), k, v)
+  inv = 1.0 / np.arange(1, S + 1)
+  ref1 = np.cumsum(inv[::-1])[::-1]
+  ref2 = np.cumsum((inv ** 2)[::-1])[::-1]
+  assert np.abs(s1[0, 1].numpy() - ref1).max() < 1e-5
+  assert np.abs(s2[0, 1].numpy() - ref2).max() < 1e-6
+  out, s1, s2 = oracle.roco_forward(q, k, v)
+  _, cs, cq, _ = brute.attention_stats(q, k, v)
+  assert (s2 >= 0).all() and (s2 <= s1 + 1e-6).all()
+  assert np.abs(s1.numpy() - cs).max() / cs.max() < 2e-3
+  assert np.abs(s2.numpy() - cq).max() / cq.max() < 4e-3
+  _, h2o = oracle.h2o_forward(q, k, v)
+  assert torch.equal(h2o, s1)
+  mean, var = oracle.roco_mean_var(s1, s2, S)
+  assert torch.allclose(mean.sum(-1), torch.ones(1, 2), rtol=1e-5) and (var > -1e-7).all()
+
+
+def test_keyformer_reductions_and_brute_force():
+  S = 64
+  q, k, v = _inputs(S=S, D=64, seed=2)
+  _, h2o = oracle.h2o_forward(q, k, v)
+  ones = torch.ones(1, 2, S, S)
+  out, kf = oracle.keyformer_forward(q, k, v, ones, tau=1.0)
+  # no noise, tau = 1: the perturbed softmax is the plain softmax
+  assert torch.allclose(kf, h2o, rtol=1e-6, atol=1e-7)
+  assert torch.equal(out, oracle.attn_forward(q, k, v))
+  # tau -> inf: uniform over the visible keys, whatever the noise
+  er = oracle.prepare_exp_rand(1, 2, S, S, seed=5)
+  _, kf_inf = oracle.keyformer_forward(q, k, v, er, tau=1e9)
+  harm = np.concatenate([[0.0], np.cumsum(1.0 / np.arange(1, S + 1))])
+  assert np.abs(kf_inf[0, 0].numpy() - (harm[S] - harm[:S])).max() < 1e-4
+  # random noise, reference default tau = 1.5, against fp64 brute force
+  _, kf = oracle.keyformer_forward(q, k, v, er)
+  _, _, _, ref = brute.attention_stats(q, k, v, exp_rand=er, tau=1.5)
+  assert np.abs(kf.numpy() - ref).max() / ref.max() < 2e-3
+  assert torch.allclose(kf.sum(-1), torch.full((1, 2), float(S)), rtol=1e-5)
+  # sign of the Gumbel term: a huge exp_rand on one key column pushes its score down
+  er2 = torch.ones(1, 2, S, S); er2[..., 3] = 1e4
+  _, kf2 = oracle.keyformer_forward(q, k, v, er2, tau=1.0)
+  assert (kf2[..., 3] < 1e-2 * h2o[..., 3]).all()
+
+
+# ------------------------------------------------------------------ linear attention
+
+def test_ea_closed_forms_and_brute_force():
+  q, k, v = _inputs(B=2, S=48, H=2, D=64, seed=4)
+  out = oracle.ea_forward(q, k, v)
+  assert out.dtype == torch.float16 and out.shape == q.shape
+  assert np.abs(out.float().numpy() - brute.ea(q, k, v)).max() < 2e-3
+  # rows of Qs and columns of Ks sum to one: constant V passes through unchanged
+  c = torch.full_like(v, 0.75)
+  assert (oracle.ea_forward(q, k, c).float() - 0.75).abs().max() < 1e-3
+  # Q = K = 0: uniform weights on both sides => every output row is the token mean of V
+  z = torch.zeros_like(q)
+  ref = v.float().mean(dim=1, keepdim=True).mean(dim=3, keepdim=True) * 0 + v.float().mean(dim=1, keepdim=True)
+  got = oracle.ea_forward(z, z, v).float()
+  # Qs uniform over D averages KV rows; Ks uniform over S makes every KV row the token mean of V
+  assert (got - ref.expand_as(got)).abs().max() < 1e-3
+
+
+def test_sima_invariants_and_brute_force():
+  q, k, v = _inputs(B=1, S=40, H=2, D=64, seed=6)
+  out32 = oracle.sima_forward(q, k, v, out_dtype=torch.float32)
+  ref = brute.sima(q, k, v)
+  assert np.abs(out32.numpy() - ref).max() / np.abs(ref).max() < 1e-5
+  raw = oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32)
+  ref_raw = brute.sima(q, k, v, normalize_q=False)
+  assert np.abs(raw.numpy() - ref_raw).max() / np.abs(ref_raw).max() < 1e-5
+  # positive rescaling of Q or K leaves the normalised form unchanged
+  out_scaled = oracle.sima_forward(q * 2, k * 0.5, v, out_dtype=torch.float32)
+  assert torch.allclose(out_scaled, out32, rtol=1e-5, atol=1e-9)
+  # K >= 0 and constant V: Kh^T V = c for every channel => O[s,e] = c * sum_d Qh[s,d]
+  kp = k.abs()
+  c = torch.full_like(v, 0.5)
+  got = oracle.sima_forward(q, kp, c, out_dtype=torch.float32)
+  qh = q.transpose(1, 2).float(); qh = qh / qh.abs().sum(dim=2, keepdim=True)
+  want = 0.5 * qh.sum(dim=3, keepdim=True).expand_as(qh).transpose(1, 2)
+  assert torch.allclose(got, want, rtol=1e-4, atol=1e-8)
+
+
+# ------------------------------------------------------------------ epilogues, recipes, chunking
+
+def test_heavy_hitters_and_gap_rule():
+  score = torch.tensor([[[0.1, 5.0, 3.0, 3.0000001, 0.2, 4.0, 0.0, 1.0]]])
+  idx = oracle.heavy_hitters(score, 3)
+  assert set(idx[0, 0].tolist()) in ({1, 5, 2}, {1, 5, 3})
+  assert oracle.topk_agreement(idx, score, 3) == 0
+  # swapping the near-tied pair is allowed, dropping a clear heavy hitter is not
+  assert oracle.topk_agreement(torch.tensor([[[1, 5, 3]]]), score, 3) == 0
+  assert oracle.topk_agreement(torch.tensor([[[1, 2, 3]]]), score, 3) == 1
+  assert oracle.topk_agreement(torch.tensor([[[1, 5, 7]]]), score, 3) == 1
+
+
+def test_chunked_over_heads_is_identical():
+  q, k, v = _inputs(B=1, S=64, H=4, D=64, seed=9)
+  full = oracle.roco_forward(q, k, v)
+  part = oracle.chunked_over_heads(oracle.roco_forward, (q, k, v), head_chunk=1)
+  for a, b in zip(full, part):
+    assert torch.equal(a, b)
+  er = oracle.prepare_exp_rand(1, 4, 64, 64)
+  full = oracle.keyformer_forward(q, k, v, er, tau=1.0)
+  part = oracle.chunked_over_heads(oracle.keyformer_forward, (q, k, v), head_chunk=2, extra=(er,), tau=1.0)
+  for a, b in zip(full, part):
+    assert torch.equal(a, b)
+
+
+def test_prepare_inputs_is_seeded_and_ordered():
+  q, k, v = oracle.prepare_inputs(1, 16, 2, 64, seed=0)
+  g = torch.Generator().manual_seed(0)
+  assert torch.equal(q, torch.randn(1, 16, 2, 64, dtype=torch.float16, generator=g))
+  assert torch.equal(k, torch.randn(1, 16, 2, 64, dtype=torch.float16, generator=g))
+  assert not torch.equal(q, oracle.prepare_inputs(1, 16, 2, 64, seed=1)[0])
+  er = oracle.prepare_exp_rand(1, 2, 16, 16)
+  assert (er >= 1).all() and er.dtype == torch.float32
+
+
+def test_reference_rounding_points():
+  # the eager definition rounds QK^T to fp16 and divides by sqrt(D) in fp16 before the fp32 softmax
+  q, k, v = _inputs(S=64, D=128, seed=11)
+  scores, probs = oracle.cases._masked_scores_probs(q, k)
+  assert scores.dtype == torch.float16 and probs.dtype == torch.float32
+  s32 = torch.matmul(q.transpose(1, 2).float(), k.transpose(1, 2).float().transpose(-2, -1))
+  manual = (s32.half().float() / torch.tensor(math.sqrt(128), dtype=torch.float32)).half()
+  tri = torch.tril(torch.ones(64, 64, dtype=torch.bool))
+  assert torch.equal(scores[..., tri], manual[..., tri])
+  assert torch.isinf(scores[..., ~tri]).all()
+
+
+# ------------------------------------------------------------------ seeded noise stream
+
+def test_noise_stream_statistics():
+  E = oracle.seeded_exp_rand(1234, 1, 2, 256, 256)
+  assert E.dtype == torch.float32 and (E > 0).all() and torch.isfinite(E).all()
+  u = torch.exp(-E.double())
+  # uniform(0,1): mean 1/2, var 1/12; Exp(1): mean 1, var 1
+  assert abs(u.mean().item() - 0.5) < 5e-3 and abs(u.var().item() - 1 / 12) < 2e-3
+  assert abs(E.mean().item() - 1.0) < 2e-2 and abs(E.var().item() - 1.0) < 5e-2
+  # Kolmogorov-Smirnov against U(0,1)
+  from scipy import stats
+  assert stats.kstest(u[0, 0].flatten().numpy()[:20000], "uniform").pvalue > 1e-3
+  # neighbouring rows / columns / heads are uncorrelated
+  x = u[0, 0] - 0.5
+  n = x.numel()
+  for a, b in ((x[1:], x[:-1]), (x[:, 1:], x[:, :-1]), (x, u[0, 1] - 0.5)):
+    corr = (a * b).mean().item() / (1 / 12)
+    assert abs(corr) < 5 / math.sqrt(n)
+  # a different seed gives a different stream; the same seed is reproducible
+  assert not torch.equal(E, oracle.seeded_exp_rand(1235, 1, 2, 256, 256))
+  assert torch.equal(E[:, :, 5:9], oracle.seeded_exp_rand(1234, 1, 2, 4, 256, row_offset=5))
+
+
+def test_lowbias32_known_answers():
+  # computed by hand-running the definition with Python integers (independent of numpy's wraparound)
+  def ref(x):
+    x &= 0xFFFFFFFF
+    x ^= x >> 16; x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15; x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return x
+  xs = [0, 1, 2, 0xFFFFFFFF, 0x12345678, 0x9E3779B9]
+  got = oracle.lowbias32(np.array(xs, dtype=np.uint64))
+  assert [int(g) for g in got] == [ref(x) for x in xs]
+  assert int(oracle.lowbias32(0)) == 0 and len(set(int(g) for g in got)) == len(xs)
