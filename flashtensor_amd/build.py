@@ -1,0 +1,65 @@
+"""Builds libflashtensor_hip.so (gfx950 only) in-tree with hipcc.
+
+    python -m flashtensor_amd.build [--force]
+
+One translation unit per kernel family, compiled in parallel, linked into a single shared library with
+the C ABI of include/ft_abi.h.  hipcc cross-compiles, so this runs on hosts without a GPU.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(CSRC, "build")
+LIB_PATH = os.path.join(HERE, "libflashtensor_hip.so")
+SOURCES = ["abi.hip", "attn_fwd.hip", "colstats.hip", "linattn.hip", "aux.hip"]
+HEADERS = ["device_common.hpp", "kernel_params.h", "noise.h", os.path.join("..", "..", "include", "ft_abi.h")]
+# packed fp32 VALU ops are disabled on purpose: some forms have produced wrong results on this hardware
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-command-line-argument"]
+
+
+def _hipcc():
+  rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+  cand = os.path.join(rocm, "bin", "hipcc")
+  return cand if os.path.exists(cand) else "hipcc"
+
+
+def _stale(target, deps):
+  if not os.path.exists(target):
+    return True
+  t = os.path.getmtime(target)
+  return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _compile(src, force):
+  obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+  deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS]
+  if not force and not _stale(obj, deps):
+    return obj, ""
+  cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+  res = subprocess.run(cmd, capture_output=True, text=True)
+  if res.returncode != 0:
+    raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")
+  return obj, res.stderr
+
+
+def build(force=False, verbose=True):
+  os.makedirs(OBJ_DIR, exist_ok=True)
+  with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+    results = list(ex.map(lambda s: _compile(s, force), SOURCES))
+  objs = [o for o, _ in results]
+  if force or _stale(LIB_PATH, objs):
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+      raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+  if verbose:
+    print(f"built {LIB_PATH}")
+  return LIB_PATH
+
+
+if __name__ == "__main__":
+  build(force="--force" in sys.argv)

@@ -1,0 +1,145 @@
+// Device-side building blocks shared by the gfx950 kernels: MFMA operand types, LDS tile staging with
+// XOR swizzles, transposed LDS reads, wave-level exchanges.
+//
+// MFMA operand layouts used throughout (v_mfma_f32_32x32x16_{f16,bf16}, wave64), lane l, g = l / 32:
+//   A (32 x 16): lane holds row l % 32, k = 8 g + [0..7]
+//   B (16 x 32): lane holds column l % 32, k = 8 g + [0..7]
+//   C (32 x 32): lane holds column l % 32, register r holds row 8 (r / 4) + 4 g + r % 4
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ft {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+#define FT_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Element traits: 16-bit storage type <-> MFMA flavour.
+struct F16 {
+  typedef half8 vec8;
+  typedef _Float16 elem;
+  static __device__ __forceinline__ elem to_elem(uint16_t bits) { return __builtin_bit_cast(_Float16, bits); }
+  static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint16_t from_float(float x) {
+    _Float16 h = (_Float16)x;
+    return __builtin_bit_cast(uint16_t, h);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t x) { return (float)__builtin_bit_cast(_Float16, x); }
+};
+struct BF16 {
+  typedef bf16x8 vec8;
+  typedef __bf16 elem;
+  static __device__ __forceinline__ elem to_elem(uint16_t bits) { return __builtin_bit_cast(__bf16, bits); }
+  static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint16_t from_float(float x) {  // round to nearest even
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
+};
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+
+// Value held by the partner lane l ^ 32 (the other 16 rows of a 32x32 accumulator column).
+__device__ __forceinline__ float xchg32(float x) { return __shfl_xor(x, 32); }
+
+__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
+
+// ---------------------------------------------------------------------------------------------------
+// A tile of ROWS x D 16-bit elements staged in LDS, rows of RB = 2 D bytes split in 16-byte chunks.
+// Two placements of chunk c of row r:
+//   kRowSwizzle : chunk index ^ ((r / RPW) % CPR)        -> conflict-free 16-byte reads of one chunk
+//                 column by 16 consecutive rows (MFMA operand with the contraction axis contiguous)
+//   kTrSwizzle  : chunk index ^ (((r / RPW) % GPR) << 2) -> conflict-free ds_read_b64_tr_b16 of 4
+//                 consecutive rows x 64 bytes (MFMA operand with the contraction axis strided)
+// RPW = rows per 256-byte bank window, CPR = chunks per row, GPR = 64-byte granules per row.
+template <int D>
+struct TileGeom {
+  static constexpr int RB = 2 * D;
+  static constexpr int CPR = RB / 16;
+  static constexpr int RPW = 256 / RB;
+  static constexpr int GPR = RB / 64;
+  static __device__ __forceinline__ int row_swz(int r) { return (r / RPW) % CPR; }
+  static __device__ __forceinline__ int tr_swz(int r) { return ((r / RPW) % GPR) << 2; }
+};
+
+enum Swizzle { kRowSwizzle = 0, kTrSwizzle = 1 };
+
+// Cooperative global -> LDS copy of a ROWS x D tile by NT threads with direct-to-LDS loads
+// (global_load_lds_dwordx4: LDS address = wave-uniform base + lane * 16).  The swizzle is applied on
+// the global side: the lane that fills LDS slot (r, c') fetches global chunk c' ^ swz(r).
+// `src` points at row 0 of the tile, `row_stride` in elements; rows >= rows_valid re-read the last valid
+// row (callers mask them).  Completion: wait_vmem() then a workgroup barrier.
+template <int D, int ROWS, int NT, int SWZ>
+__device__ __forceinline__ void stage_tile(const uint16_t* __restrict__ src, int64_t row_stride, int rows_valid,
+                                           char* lds_tile) {
+  typedef TileGeom<D> G;
+  constexpr int CHUNKS = ROWS * G::CPR;
+  static_assert(CHUNKS % NT == 0, "tile must be a whole number of rounds");
+  const int lane = lane_id();
+  const int wave = wave_id();
+#pragma unroll
+  for (int it = 0; it < CHUNKS / NT; ++it) {
+    const int slot = it * NT + wave * 64 + lane;  // 16-byte slot index in the tile
+    const int r = slot / G::CPR;
+    const int cs = slot % G::CPR;
+    const int c = cs ^ (SWZ == kRowSwizzle ? G::row_swz(r) : G::tr_swz(r));
+    const int rr = r < rows_valid ? r : rows_valid - 1;
+    const uint16_t* g = src + (int64_t)rr * row_stride + c * 8;
+    char* dst = lds_tile + (it * NT + wave * 64) * 16;  // wave-uniform
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, FT_LDS(void, dst), 16, 0, 0);
+  }
+}
+
+// 8 contiguous elements (one 16-byte chunk `c`) of row `r` from a kRowSwizzle tile.
+template <int D, typename V8>
+__device__ __forceinline__ V8 read_row_chunk(const char* lds_tile, int r, int c) {
+  typedef TileGeom<D> G;
+  return *reinterpret_cast<const V8*>(lds_tile + r * G::RB + ((c ^ G::row_swz(r)) << 4));
+}
+
+// Transposed operand from a kTrSwizzle tile: the calling lane (column d = d_base + l % 32 of the tile,
+// g = l / 32) receives rows {k0 + 4 g + [0..3], k0 + 8 + 4 g + [0..3]} of that column: the 8
+// contraction slots that pair with registers [rb .. rb+7] of a 32x32 accumulator whose rows start at k0.
+// ds_read_b64_tr_b16: within each 16-lane group, lane i receives element i % 4 of the 8-byte rows
+// addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4.
+template <int D, typename V8>
+__device__ __forceinline__ V8 read_tr_operand(const char* lds_tile, int k0, int d_base) {
+  typedef TileGeom<D> G;
+  const int l = lane_id();
+  const int j16 = l & 15;
+  const int dhalf = (l >> 4) & 1;
+  const int g = l >> 5;
+  const int d0 = d_base + 16 * dhalf + 4 * (j16 & 3);
+  const int r0 = k0 + 4 * g + (j16 >> 2);
+  const int r1 = r0 + 8;
+  const int c = d0 >> 3;
+  const int within = (d0 & 7) * 2;
+  const char* p0 = lds_tile + r0 * G::RB + ((c ^ G::tr_swz(r0)) << 4) + within;
+  const char* p1 = lds_tile + r1 * G::RB + ((c ^ G::tr_swz(r1)) << 4) + within;
+  short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(FT_LDS(short4v, p0));
+  short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(FT_LDS(short4v, p1));
+  short8v both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(V8, both);
+}
+
+}  // namespace ft

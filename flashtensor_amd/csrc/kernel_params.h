@@ -1,0 +1,48 @@
+// Launch-time parameter blocks shared by the host dispatcher and the kernels.
+#pragma once
+#include <stdint.h>
+
+namespace ft {
+
+struct Strides3 {
+  int64_t b, s, h;
+};
+
+struct AttnKernelParams {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  uint16_t* o;
+  Strides3 sq, sk, sv, so;
+  float* lse;     // [B,H,Sq] log2-domain normaliser of the plain softmax (may be null)
+  float* lse_kf;  // [B,H,Sq] normaliser of the perturbed softmax (KeyFormer modes)
+  const float* exp_rand;
+  int64_t er_sb, er_sh, er_sr;
+  int er_vec4;  // exp_rand rows can be read as aligned float4
+  uint64_t seed;
+  int B, H, Sq, Skv;
+  int off;          // Skv - Sq: query i sees keys j <= i + off when causal
+  float logit_mul;  // reference rounding: f16(f16(acc) * logit_mul) == f16(f16(acc) / sqrt(D)); fast: log2e / sqrt(D)
+  float inv_tau;
+};
+
+struct ColstatsKernelParams {
+  const uint16_t* q;
+  const uint16_t* k;
+  Strides3 sq, sk;
+  const float* lse;  // [B,H,Sq] normaliser of the distribution being summed
+  float* colsum;     // [B,H,Skv]
+  float* colsumsq;   // [B,H,Skv] or null
+  const float* exp_rand;
+  int64_t er_sb, er_sh, er_sr;
+  uint64_t seed;
+  int B, H, Sq, Skv;
+  int off;
+  float logit_mul;
+  float inv_tau;
+};
+
+enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2 };
+enum StatMode { kStatSum = 0, kStatSumSq = 1, kStatKfTensor = 2, kStatKfSeeded = 3 };
+
+}  // namespace ft

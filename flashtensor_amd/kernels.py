@@ -1,0 +1,125 @@
+"""Case modules with the interface of the reference's workload zoo (cases/kernels/*.py): a class per
+workload with `forward(...)` returning the same tensors in the same order, `prepare(...)` returning the
+`{'input': {...}, 'output': [...]}` recipe, and `get_model()`.  `forward` runs the fused HIP kernels.
+"""
+import torch
+
+from . import ops
+
+
+class _Case:
+  output = []
+
+  def __init__(self, kv_head_num=32, head_num=32, head_dim=128):
+    self.kv_head_num = kv_head_num
+    self.head_num = head_num
+    self.head_dim = head_dim
+    self.hidden_size = head_num * head_dim
+    self.kv_hidden_size = kv_head_num * head_dim
+    self.group_size = self.head_num // self.kv_head_num
+    assert self.group_size == 1  # as cases/kernels/attn.py:16
+
+  def __call__(self, *args):
+    return self.forward(*args)
+
+  def eval(self):
+    return self
+
+  def _qkv(self, batch_size, q_len, kv_len, dtype, device):
+    q = torch.randn(batch_size, q_len, self.head_num, self.head_dim, dtype=dtype, device=device)
+    k = torch.randn(batch_size, kv_len, self.head_num, self.head_dim, dtype=dtype, device=device)
+    v = torch.randn(batch_size, kv_len, self.head_num, self.head_dim, dtype=dtype, device=device)
+    return {"q": q, "k": k, "v": v}
+
+  def prepare(self, batch_size=1, q_len=4096, kv_len=4096, dtype=torch.float16, device=None):
+    """Input recipe of cases/kernels/attn.py:36-49 (defaults B=1, S=4096, fp16, current GPU)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    return {"input": self._qkv(batch_size, q_len, kv_len, dtype, device), "output": list(self.output)}
+
+
+class Attn(_Case):
+  """cases/kernels/attn.py: out = softmax(QK^T/sqrt(D) + causal) V."""
+  output = ["out"]
+
+  def forward(self, q, k, v):
+    return ops.attn(q, k, v)
+
+
+class H2O(_Case):
+  """cases/kernels/h2o.py: (out, h2o_score)."""
+  output = ["out", "h2o_score"]
+
+  def forward(self, q, k, v):
+    return ops.h2o(q, k, v)
+
+  def heavy_hitters(self, h2o_score, k=None):
+    """Top-k key indices per head (k defaults to S/8)."""
+    return ops.topk(h2o_score, k or h2o_score.shape[-1] // 8)
+
+
+class RoCo(_Case):
+  """cases/kernels/roco.py: (out, roco_score, roco_sq_score)."""
+  output = ["out", "roco_score", "roco_sq_score"]
+
+  def forward(self, q, k, v):
+    return ops.roco(q, k, v)
+
+  @staticmethod
+  def mean_var(roco_score, roco_sq_score, q_len):
+    mean = roco_score / q_len
+    return mean, roco_sq_score / q_len - mean * mean
+
+
+class KeyFormer(_Case):
+  """cases/kernels/kf.py: (out, kf_score); tau defaults to 1.5 as kf.py:8.  Passing exp_rand=None to
+  forward draws the noise in-kernel from `seed`."""
+  output = ["out", "kf_score"]
+
+  def __init__(self, tau=1.5, kv_head_num=32, head_num=32, head_dim=128, seed=0):
+    super().__init__(kv_head_num, head_num, head_dim)
+    self.tau = tau
+    self.seed = seed
+
+  def forward(self, q, k, v, exp_rand=None):
+    return ops.keyformer(q, k, v, exp_rand, tau=self.tau, seed=self.seed)
+
+  def prepare(self, batch_size=1, q_len=4096, kv_len=4096, dtype=torch.float16, device=None):
+    ret = super().prepare(batch_size, q_len, kv_len, dtype, device)
+    dev = ret["input"]["q"].device
+    ret["input"]["exp_rand"] = 1 + torch.randn(batch_size, self.head_num, q_len, kv_len, dtype=torch.float32, device=dev).abs()
+    return ret
+
+
+class EA(_Case):
+  """Attention core of bench/ea.mlir:13-17 on [B,S,H,D] tensors."""
+  output = ["out"]
+
+  def __init__(self, kv_head_num=16, head_num=16, head_dim=64):
+    super().__init__(kv_head_num, head_num, head_dim)
+
+  def forward(self, q, k, v):
+    return ops.ea(q, k, v)
+
+  def prepare(self, batch_size=8, q_len=8192, kv_len=None, dtype=torch.float16, device=None):
+    return super().prepare(batch_size, q_len, q_len, dtype, device)
+
+
+class SimA(EA):
+  """Attention core of bench/sima.mlir:13-17 on [B,S,H,D] tensors."""
+
+  def __init__(self, kv_head_num=16, head_num=16, head_dim=64, normalize_q=True):
+    super().__init__(kv_head_num, head_num, head_dim)
+    self.normalize_q = normalize_q
+
+  def forward(self, q, k, v):
+    return ops.sima(q, k, v, normalize_q=self.normalize_q)
+
+
+CASES = {"attn": Attn, "h2o": H2O, "kf": KeyFormer, "roco": RoCo, "ea": EA, "sima": SimA}
+
+
+def get_model(name="attn", **kw):
+  """`importlib.import_module('.' + name, 'kernels').get_model()` of cases/run.py:15-16, as one call."""
+  if name not in CASES:
+    raise KeyError(f"unknown case {name!r}; have {sorted(CASES)}")
+  return CASES[name](**kw)

@@ -1,0 +1,175 @@
+"""Torch-facing operators over the C ABI: one function per fused workload.
+
+Call convention of the reference's emitted kernel wrapper (lib/Translate/to_triton.cpp:540-609): positional
+torch tensors in, results allocated with torch.empty on the device of the first argument and returned
+(a tuple when there are several), launch on the current stream, no synchronisation.  Torch is used for
+device memory and the stream handle only; all arithmetic happens in libflashtensor_hip.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import FtAttnArgs, FtNoise, FtStrides
+
+_DTYPES = {torch.float16: _lib.FT_F16, torch.bfloat16: _lib.FT_BF16}
+
+
+def _stream(t):
+  return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _check_qkv(q, k, v):
+  for i, t in enumerate((q, k, v)):
+    if not isinstance(t, torch.Tensor):
+      raise RuntimeError(f"arg {i} need a torch.Tensor but got {type(t).__name__}")
+    if t.dim() != 4:
+      raise RuntimeError(f"arg {i} need shape [B, S, H, D] but got {tuple(t.shape)}")
+    if not t.is_cuda:
+      raise RuntimeError(f"arg {i} need a GPU tensor but got device {t.device}")
+    if t.dtype != q.dtype or t.device != q.device:
+      raise RuntimeError(f"arg {i} need dtype {q.dtype} on {q.device} but got {t.dtype} on {t.device}")
+  if q.dtype not in _DTYPES:
+    raise RuntimeError(f"arg 0 need dtype float16 or bfloat16 but got {q.dtype}")
+  B, Sq, H, D = q.shape
+  if tuple(k.shape) != (B, k.shape[1], H, D):
+    raise RuntimeError(f"arg 1 need shape {(B, k.shape[1], H, D)} but got {tuple(k.shape)}")
+  if tuple(v.shape) != tuple(k.shape):
+    raise RuntimeError(f"arg 2 need shape {tuple(k.shape)} but got {tuple(v.shape)}")
+
+
+def _dense_last(t):
+  return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _strides(t):
+  return FtStrides(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _args(q, k, v, o, flags):
+  B, Sq, H, D = q.shape
+  return FtAttnArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _strides(q), _strides(k), _strides(v),
+                    _strides(o), B, H, Sq, k.shape[1], D, _DTYPES[q.dtype], flags)
+
+
+def _flags(causal, fast_logits):
+  return (_lib.FT_CAUSAL if causal else 0) | (_lib.FT_FAST_LOGITS if fast_logits else 0)
+
+
+def _prep(q, k, v):
+  _check_qkv(q, k, v)
+  return _dense_last(q), _dense_last(k), _dense_last(v)
+
+
+def attn(q, k, v, causal=True, fast_logits=False, return_lse=False):
+  """Attn.forward (cases/kernels/attn.py:18-34): q,k,v [B,S,H,D] -> out [B,Sq,H,D]."""
+  q, k, v = _prep(q, k, v)
+  lib = _lib.load()
+  out = torch.empty_like(q, memory_format=torch.contiguous_format)
+  lse = torch.empty(q.shape[0], q.shape[2], q.shape[1], dtype=torch.float32, device=q.device) if return_lse else None
+  a = _args(q, k, v, out, _flags(causal, fast_logits))
+  _lib.check(lib.ft_attn_fwd(ctypes.byref(a), lse.data_ptr() if return_lse else None, _stream(q)))
+  return (out, lse) if return_lse else out
+
+
+def _colstats(q, k, v, want_sq, causal, fast_logits):
+  q, k, v = _prep(q, k, v)
+  lib = _lib.load()
+  B, Sq, H, D = q.shape
+  Skv = k.shape[1]
+  out = torch.empty_like(q, memory_format=torch.contiguous_format)
+  s1 = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device)
+  s2 = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device) if want_sq else None
+  a = _args(q, k, v, out, _flags(causal, fast_logits))
+  nbytes = lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a))
+  ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+  _lib.check(lib.ft_attn_colstats_fwd(ctypes.byref(a), s1.data_ptr(), s2.data_ptr() if want_sq else None,
+                                      ws.data_ptr(), nbytes, _stream(q)))
+  return (out, s1, s2) if want_sq else (out, s1)
+
+
+def h2o(q, k, v, causal=True, fast_logits=False):
+  """H2O.forward (cases/kernels/h2o.py:18-38) -> (out, h2o_score [B,H,Skv] fp32)."""
+  return _colstats(q, k, v, False, causal, fast_logits)
+
+
+def roco(q, k, v, causal=True, fast_logits=False):
+  """RoCo.forward (cases/kernels/roco.py:18-48) -> (out, roco_score, roco_sq_score), scores [B,H,Skv] fp32."""
+  return _colstats(q, k, v, True, causal, fast_logits)
+
+
+def keyformer(q, k, v, exp_rand=None, tau=1.5, seed=0, causal=True, fast_logits=False):
+  """KeyFormer.forward (cases/kernels/kf.py:19-42) -> (out, kf_score [B,H,Skv] fp32).
+  exp_rand [B,H,Sq,Skv] fp32 is the reference's noise input; None draws it in-kernel from `seed`."""
+  q, k, v = _prep(q, k, v)
+  lib = _lib.load()
+  B, Sq, H, D = q.shape
+  Skv = k.shape[1]
+  noise = FtNoise(None, 0, 0, 0, int(seed) & 0xFFFFFFFFFFFFFFFF)
+  if exp_rand is not None:
+    if tuple(exp_rand.shape) != (B, H, Sq, Skv):
+      raise RuntimeError(f"arg 3 need shape {(B, H, Sq, Skv)} but got {tuple(exp_rand.shape)}")
+    if exp_rand.dtype != torch.float32 or exp_rand.device != q.device:
+      raise RuntimeError(f"arg 3 need dtype torch.float32 on {q.device} but got {exp_rand.dtype} on {exp_rand.device}")
+    exp_rand = _dense_last(exp_rand)
+    noise = FtNoise(exp_rand.data_ptr(), exp_rand.stride(0), exp_rand.stride(1), exp_rand.stride(2), 0)
+  out = torch.empty_like(q, memory_format=torch.contiguous_format)
+  score = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device)
+  a = _args(q, k, v, out, _flags(causal, fast_logits))
+  nbytes = lib.ft_workspace_bytes(_lib.FT_OP_KEYFORMER, ctypes.byref(a))
+  ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+  _lib.check(lib.ft_keyformer_fwd(ctypes.byref(a), ctypes.byref(noise), float(tau), score.data_ptr(), ws.data_ptr(),
+                                  nbytes, _stream(q)))
+  return out, score
+
+
+def _linattn(q, k, v, kind, normalize_q, out_dtype):
+  q, k, v = _prep(q, k, v)
+  lib = _lib.load()
+  out_dtype = out_dtype or q.dtype
+  if out_dtype not in (torch.float16, torch.float32):
+    raise RuntimeError(f"out_dtype need float16 or float32 but got {out_dtype}")
+  out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+  a = _args(q, k, v, out, 0)
+  nbytes = lib.ft_workspace_bytes(kind, ctypes.byref(a))
+  ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+  _lib.check(lib.ft_linattn_fwd(ctypes.byref(a), kind, int(bool(normalize_q)),
+                                _lib.FT_F32 if out_dtype == torch.float32 else _lib.FT_F16, ws.data_ptr(), nbytes, _stream(q)))
+  return out
+
+
+def ea(q, k, v, out_dtype=None):
+  """EA core (bench/ea.mlir:13-17): softmax(Q, dim=D) (softmax(K, dim=S)^T V); q,k,v [B,S,H,D] -> [B,S,H,D]."""
+  return _linattn(q, k, v, _lib.FT_OP_EA, True, out_dtype)
+
+
+def sima(q, k, v, normalize_q=True, out_dtype=None):
+  """SimA core (bench/sima.mlir:13-17): L1-normalised Q, K over S per channel, O = Qh (Kh^T V).
+  normalize_q=False multiplies by the raw Q as line 17 of the .mlir does."""
+  return _linattn(q, k, v, _lib.FT_OP_SIMA, normalize_q, out_dtype)
+
+
+def topk(score, k):
+  """Indices [..., k] (int64) of the k largest entries along the last axis, descending."""
+  if score.dtype != torch.float32 or not score.is_cuda:
+    raise RuntimeError(f"arg 0 need a float32 GPU tensor but got {score.dtype} on {score.device}")
+  lib = _lib.load()
+  s = score.contiguous()
+  S = s.shape[-1]
+  rows = s.numel() // S
+  idx = torch.empty(*s.shape[:-1], k, dtype=torch.int64, device=s.device)
+  _lib.check(lib.ft_topk(s.data_ptr(), rows, S, int(k), idx.data_ptr(), _stream(s)))
+  return idx
+
+
+def seeded_exp_rand(B, H, Sq, Skv, seed, device):
+  """The noise tensor the seeded KeyFormer mode draws, materialised on `device` ("cpu" uses the host twin)."""
+  lib = _lib.load()
+  device = torch.device(device)
+  out = torch.empty(B, H, Sq, Skv, dtype=torch.float32, device=device)
+  seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+  if device.type == "cpu":
+    _lib.check(lib.ft_noise_exp_fill_host(out.data_ptr(), B, H, Sq, Skv, seed))
+  else:
+    _lib.check(lib.ft_noise_exp_fill(out.data_ptr(), B, H, Sq, Skv, seed, _stream(out)))
+  return out

@@ -1,0 +1,113 @@
+/*
+ * C ABI of libflashtensor_hip: fused attention-variant kernels for AMD MI355X (gfx950).
+ *
+ * This is the boundary a host program binds (ctypes, pybind11, cgo ...): plain pointers, sizes and
+ * POD structs only.  Every function returns FT_OK (0) or a negative FT_E* code; ft_last_error() then
+ * holds a thread-local message.  Device pointers are borrowed for the duration of the call, nothing
+ * is retained, no device memory is allocated or freed, and no call synchronises: kernels are queued
+ * on the hipStream_t passed as `stream` (NULL = the null stream).
+ *
+ * What each entry point replaces in the reference (monellz/FlashTensor):
+ *   the emitted kernel wrapper `def <Kernel>(arg0: torch.Tensor, ...) -> Tuple[...]` that allocates the
+ *   results and launches the fused Triton kernel (lib/Translate/to_triton.cpp:529-638, device kernel
+ *   :480-527), and the TensorRT closure used by the harnesses
+ *   (python/asuka/backend/tensorrt/builder.py:73-151), for the workloads defined in
+ *   cases/kernels/{attn,h2o,kf,roco}.py and bench/{ea,sima}.mlir.
+ */
+#ifndef FT_ABI_H
+#define FT_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FT_ABI_VERSION 1
+
+enum FtStatus {
+  FT_OK = 0,
+  FT_EINVAL = -1,       /* bad argument (null pointer, shape, stride, alignment) */
+  FT_EUNSUPPORTED = -2, /* valid request the kernels do not cover (head_dim, dtype, ...) */
+  FT_ELAUNCH = -3,      /* HIP reported an error at launch */
+  FT_EWORKSPACE = -4    /* workspace missing or smaller than ft_workspace_bytes() */
+};
+
+enum FtDtype { FT_F16 = 0, FT_BF16 = 1, FT_F32 = 2 };
+
+enum FtFlags {
+  FT_CAUSAL = 1u,      /* mask key j for query i when j > i + (Skv - Sq)  (cases/kernels/attn.py:22-23) */
+  FT_FAST_LOGITS = 2u  /* keep QK^T/sqrt(D) in fp32 instead of reproducing the reference's fp16 rounding
+                          of the logits (cases/kernels/attn.py:29); faster, ~1e-3 relative on probabilities */
+};
+
+enum FtOp { FT_OP_ATTN = 0, FT_OP_COLSTATS = 1, FT_OP_KEYFORMER = 2, FT_OP_EA = 3, FT_OP_SIMA = 4 };
+
+/* Element strides of a logical [B, S, H, D] tensor; the D axis must be contiguous (stride 1). */
+typedef struct FtStrides {
+  int64_t b, s, h;
+} FtStrides;
+
+/* One attention problem: q [B,Sq,H,D], k,v [B,Skv,H,D], o [B,Sq,H,D] (cases/kernels/attn.py:37-39, :32-34). */
+typedef struct FtAttnArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  FtStrides sq, sk, sv, so;
+  int32_t B, H, Sq, Skv, D;
+  int32_t dtype;  /* FtDtype of q, k, v, o */
+  uint32_t flags; /* FtFlags */
+} FtAttnArgs;
+
+/* KeyFormer noise source.  exp_rand != NULL: the reference's input tensor [B,H,Sq,Skv] fp32
+ * (cases/kernels/kf.py:19,36-37) with the given element strides (last axis contiguous).
+ * exp_rand == NULL: drawn in-kernel from the counter-based stream keyed by `seed`
+ * (ft_noise_exp_fill* materialise the same tensor). */
+typedef struct FtNoise {
+  const float* exp_rand;
+  int64_t stride_b, stride_h, stride_row;
+  uint64_t seed;
+} FtNoise;
+
+int ft_abi_version(void);
+const char* ft_last_error(void);
+
+/* Bytes of device scratch the op needs for this problem (0 if none).  The caller owns the buffer. */
+size_t ft_workspace_bytes(int op, const FtAttnArgs* a);
+
+/* Causal (or full) softmax attention: replaces the fused kernel of Attn.forward (cases/kernels/attn.py:18-34).
+ * lse: optional [B,H,Sq] fp32 output, log2-domain row normaliser max + log2(sum). */
+int ft_attn_fwd(const FtAttnArgs* a, float* lse, void* stream);
+
+/* Attention + per-key column statistics: H2O.forward (cases/kernels/h2o.py:18-38; colsumsq == NULL) and
+ * RoCo.forward (cases/kernels/roco.py:18-48).  colsum, colsumsq: [B,H,Skv] fp32. */
+int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+/* KeyFormer.forward (cases/kernels/kf.py:19-42): attention + column sums of softmax((logits + gumbel)/tau),
+ * gumbel = -log(exp_rand).  kf_score: [B,H,Skv] fp32. */
+int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float* kf_score, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+/* Linear attention cores of bench/ea.mlir:13-17 (kind = FT_OP_EA) and bench/sima.mlir:13-17 (FT_OP_SIMA):
+ * O = f(Q) (g(K)^T V).  normalize_q applies SimA's L1 normalisation to Q as well (ignored for EA).
+ * out_dtype: FtDtype of o (FT_F16/FT_BF16 = a->dtype, or FT_F32). */
+int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/* Heavy hitters: indices of the k largest entries of each row of score [rows, S] fp32, in descending
+ * score order (ties: lower index first), written as int64 [rows, k].  Not in the reference, whose H2O
+ * case ends at the score (cases/kernels/h2o.py:34-38); S <= 8192. */
+int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx, void* stream);
+
+/* The tensor E[B,H,Sq,Skv] = -ln(u) drawn by the seeded KeyFormer mode, written to device memory
+ * (ft_noise_exp_fill) or host memory (ft_noise_exp_fill_host). */
+int ft_noise_exp_fill(float* dst, int32_t B, int32_t H, int32_t Sq, int32_t Skv, uint64_t seed, void* stream);
+int ft_noise_exp_fill_host(float* dst, int32_t B, int32_t H, int32_t Sq, int32_t Skv, uint64_t seed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FT_ABI_H */
