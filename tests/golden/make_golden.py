@@ -1,0 +1,48 @@
+"""Writes the golden vectors of tests/golden/*.npz from the CPU oracle.
+
+    python tests/golden/make_golden.py
+
+The reference ships no fixtures for this path, so these are regression vectors of the pinned oracle
+(tests/test_oracle_pins.py): inputs are regenerated from the seed by oracle.prepare_inputs and are not
+stored; the files hold the expected outputs only (fp16 O, fp32 scores, top-k indices).
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+import oracle  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+# (name, B, S, H, D, seed)
+SHAPES = [("s128_d128", 1, 128, 2, 128, 0), ("s256_d64", 1, 256, 2, 64, 0), ("s200_d128", 1, 200, 2, 128, 1)]
+LIN_SHAPES = [("s256_d64", 1, 256, 2, 64, 0), ("s200_d64", 2, 200, 2, 64, 1)]
+KF_SEED = 1234
+
+
+def main():
+  torch.set_num_threads(1)  # fixed reduction order
+  for name, B, S, H, D, seed in SHAPES:
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+    out, s1, s2 = oracle.roco_forward(q, k, v)
+    er = oracle.prepare_exp_rand(B, H, S, S, seed=seed)
+    _, kf_t = oracle.keyformer_forward(q, k, v, er, tau=1.5)
+    _, kf_s = oracle.keyformer_forward(q, k, v, oracle.seeded_exp_rand(KF_SEED, B, H, S, S), tau=1.0)
+    np.savez_compressed(os.path.join(HERE, f"softmax_{name}.npz"), B=B, S=S, H=H, D=D, seed=seed, kf_seed=KF_SEED,
+                        out=out.numpy(), colsum=s1.numpy(), colsumsq=s2.numpy(), kf_tensor_tau15=kf_t.numpy(),
+                        kf_seeded_tau1=kf_s.numpy(), topk=oracle.heavy_hitters(s1, S // 8).numpy())
+  for name, B, S, H, D, seed in LIN_SHAPES:
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+    np.savez_compressed(os.path.join(HERE, f"linear_{name}.npz"), B=B, S=S, H=H, D=D, seed=seed,
+                        ea=oracle.ea_forward(q, k, v).numpy(),
+                        sima=oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy(),
+                        sima_rawq=oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32).numpy())
+  print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
+
+
+if __name__ == "__main__":
+  main()

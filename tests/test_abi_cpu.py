@@ -1,0 +1,122 @@
+"""The C ABI without a GPU: the library loads, exports exactly what include/ft_abi.h declares, and
+rejects bad arguments before anything is launched.  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import flashtensor_amd as ft
+from flashtensor_amd import _lib
+from flashtensor_amd._lib import FtAttnArgs, FtNoise, FtStrides
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+  return _lib.load()
+
+
+def _declared():
+  text = open(os.path.join(ROOT, "include", "ft_abi.h")).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\b(ft_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+  declared = _declared()
+  assert declared == sorted(_lib.EXPORTS)
+  for name in declared:
+    assert getattr(lib, name) is not None
+  assert lib.ft_abi_version() == 1
+
+
+def _args(**over):
+  st = FtStrides(8 * 2 * 128, 2 * 128, 128)
+  base = dict(q=0x1000, k=0x2000, v=0x3000, o=0x4000, sq=st, sk=st, sv=st, so=st, B=1, H=2, Sq=8, Skv=8, D=128,
+              dtype=_lib.FT_F16, flags=_lib.FT_CAUSAL)
+  base.update(over)
+  return FtAttnArgs(**base)
+
+
+@pytest.mark.parametrize("over,code,needle", [
+    (dict(q=None), _lib.FT_EINVAL, "null"),
+    (dict(o=None), _lib.FT_EINVAL, "null"),
+    (dict(D=96), _lib.FT_EUNSUPPORTED, "head_dim"),
+    (dict(dtype=_lib.FT_F32), _lib.FT_EUNSUPPORTED, "dtype"),
+    (dict(Sq=0), _lib.FT_EINVAL, "shape"),
+    (dict(Sq=16, Skv=8), _lib.FT_EINVAL, "Skv >= Sq"),
+    (dict(q=0x1004), _lib.FT_EINVAL, "aligned"),
+    (dict(sq=FtStrides(2048, 250, 128)), _lib.FT_EINVAL, "strides"),
+])
+def test_attn_rejects_bad_arguments_before_launch(lib, over, code, needle):
+  a = _args(**over)
+  assert lib.ft_attn_fwd(ctypes.byref(a), None, None) == code
+  assert needle in lib.ft_last_error().decode()
+  with pytest.raises((ValueError, _lib.FtError)):
+    _lib.check(code)
+
+
+def test_colstats_and_keyformer_argument_checks(lib):
+  a = _args()
+  need = lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a))
+  assert need == 1 * 2 * 8 * 4 == lib.ft_workspace_bytes(_lib.FT_OP_KEYFORMER, ctypes.byref(a))
+  assert lib.ft_workspace_bytes(_lib.FT_OP_ATTN, ctypes.byref(a)) == 0
+  assert lib.ft_attn_colstats_fwd(ctypes.byref(a), None, None, 0x5000, need, None) == _lib.FT_EINVAL
+  assert lib.ft_attn_colstats_fwd(ctypes.byref(a), 0x6000, None, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
+  assert "workspace" in lib.ft_last_error().decode()
+  assert lib.ft_attn_colstats_fwd(ctypes.byref(a), 0x6000, None, None, need, None) == _lib.FT_EWORKSPACE
+  noise = FtNoise(None, 0, 0, 0, 1)
+  assert lib.ft_keyformer_fwd(ctypes.byref(a), None, 1.0, 0x6000, 0x5000, need, None) == _lib.FT_EINVAL
+  assert lib.ft_keyformer_fwd(ctypes.byref(a), ctypes.byref(noise), 0.0, 0x6000, 0x5000, need, None) == _lib.FT_EINVAL
+  assert "tau" in lib.ft_last_error().decode()
+  assert lib.ft_keyformer_fwd(ctypes.byref(a), ctypes.byref(noise), 1.0, None, 0x5000, need, None) == _lib.FT_EINVAL
+
+
+def test_linattn_and_topk_argument_checks(lib):
+  st = FtStrides(64 * 2 * 64, 2 * 64, 64)
+  a = _args(D=64, Sq=64, Skv=64, sq=st, sk=st, sv=st, so=st, flags=0)
+  need = lib.ft_workspace_bytes(_lib.FT_OP_EA, ctypes.byref(a))
+  assert need > 0 and need % 256 == 0
+  assert lib.ft_linattn_fwd(ctypes.byref(a), 7, 1, _lib.FT_F16, 0x5000, need, None) == _lib.FT_EINVAL
+  assert lib.ft_linattn_fwd(ctypes.byref(a), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
+  b = _args(D=128, flags=0)
+  assert lib.ft_linattn_fwd(ctypes.byref(b), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EUNSUPPORTED
+  c = _args(D=64, Sq=64, Skv=32, sq=st, sk=st, sv=st, so=st, flags=0)
+  assert lib.ft_linattn_fwd(ctypes.byref(c), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EINVAL
+  assert lib.ft_topk(None, 1, 8, 2, 0x1000, None) == _lib.FT_EINVAL
+  assert lib.ft_topk(0x1000, 1, 8, 9, 0x2000, None) == _lib.FT_EINVAL
+  assert lib.ft_topk(0x1000, 1, 16384, 9, 0x2000, None) == _lib.FT_EUNSUPPORTED
+
+
+def test_host_noise_twin_matches_oracle_stream(lib):
+  import oracle
+  E = ft.ops.seeded_exp_rand(2, 3, 17, 33, 987654321987, "cpu")
+  ref = oracle.seeded_exp_rand(987654321987, 2, 3, 17, 33)
+  assert torch.allclose(E, ref, rtol=1e-6, atol=0)
+
+
+def test_operator_layer_validates_like_the_reference_backend():
+  q = torch.zeros(1, 8, 2, 128, dtype=torch.float16)
+  with pytest.raises(RuntimeError, match="need a GPU tensor"):
+    ft.ops.attn(q, q, q)
+  with pytest.raises(RuntimeError, match="need shape"):
+    ft.ops.attn(q[0], q[0], q[0])
+  with pytest.raises(KeyError):
+    ft.HipBuilder("nope")
+  f = ft.HipBuilder("h2o").build_callable()
+  with pytest.raises(RuntimeError, match="arg 0 need shape"):
+    f(torch.zeros(1, 8, 2, 64, dtype=torch.float16), q, q)
+  assert sorted(ft.CASES) == ["attn", "ea", "h2o", "kf", "roco", "sima"]
+  assert ft.get_model("kf").tau == 1.5 and ft.get_model("h2o").prepare.__doc__
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+  monkeypatch.setattr(_lib, "_lib", None)
+  monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libflashtensor_hip.so"))
+  with pytest.raises(ImportError, match="not found"):
+    _lib.load()
+  with pytest.raises(ImportError):
+    ft.HipBuilder("attn").build_callable()

@@ -1,0 +1,312 @@
+"""Parity of the HIP kernels (called through the C ABI) with the CPU oracle on the same seeded inputs.
+
+Tolerances (the stated bar for this path):
+  fp16 O        max-abs <= 2e-2 and relative (Frobenius) <= 1e-2; also a tight elementwise bound
+                |d| <= 4e-3 + 1e-2 |ref| that the kernels meet in practice
+  fp32 scores   elementwise relative <= 1e-3
+  top-k         identical index sets wherever the score gap exceeds the score tolerance
+Full-size configurations are checked against the oracle on a subset of heads (heads are independent)
+and through size-independent properties (row sums, closed forms, degenerate-noise identities).
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle.metrics import rel_fro
+import flashtensor_amd as ft
+from flashtensor_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+O_ABS, O_REL, SCORE_REL = 2e-2, 1e-2, 1e-3
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def check_o(out, ref, abs_tol=O_ABS, tight=4e-3):
+  out, ref = out.float().cpu(), ref.float()
+  d = (out - ref).abs()
+  assert torch.isfinite(out).all()
+  assert d.max().item() <= abs_tol, f"O max-abs {d.max().item()}"
+  assert rel_fro(out, ref) <= O_REL, f"O rel-fro {rel_fro(out, ref)}"
+  assert (d <= tight + O_REL * ref.abs()).all(), f"O elementwise: worst {d.max().item()}"
+
+
+def check_score(s, ref, rel=SCORE_REL):
+  s, ref = s.float().cpu(), ref.float()
+  assert torch.isfinite(s).all()
+  err = ((s - ref).abs() / ref.abs().clamp_min(1e-30)).max().item()
+  assert err <= rel, f"score rel {err}"
+
+
+def gpu_inputs(gpu, *a, **kw):
+  q, k, v = oracle.prepare_inputs(*a, **kw)
+  return (q, k, v), (q.to(gpu), k.to(gpu), v.to(gpu))
+
+
+SMALL = [(1, 128, 2, 128, 0), (1, 256, 2, 64, 1), (2, 200, 3, 128, 2), (1, 64, 1, 128, 3), (1, 1, 2, 64, 4),
+         (1, 333, 2, 64, 5), (1, 130, 2, 128, 6)]
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", SMALL)
+def test_attn_small(gpu, B, S, H, D, seed):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  out = ops.attn(qd, kd, vd)
+  check_o(out, oracle.attn_forward(q, k, v))
+  assert torch.equal(out[:, 0].cpu(), v[:, 0])  # row 0 attends to key 0 only
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", SMALL)
+def test_h2o_roco_small(gpu, B, S, H, D, seed):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  ref_o, r1, r2 = oracle.roco_forward(q, k, v)
+  out, s1, s2 = ops.roco(qd, kd, vd)
+  check_o(out, ref_o); check_score(s1, r1); check_score(s2, r2)
+  out_h, sh = ops.h2o(qd, kd, vd)
+  assert torch.equal(out_h, out) and torch.equal(sh, s1)
+  assert s1.shape == (B, H, S) and s1.dtype == torch.float32
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", SMALL[:4] + SMALL[5:])
+@pytest.mark.parametrize("tau", [1.0, 1.5])
+def test_keyformer_small(gpu, B, S, H, D, seed, tau):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  er = oracle.prepare_exp_rand(B, H, S, S, seed=seed)
+  ref_o, ref_s = oracle.keyformer_forward(q, k, v, er, tau=tau)
+  out, s = ops.keyformer(qd, kd, vd, er.to(gpu), tau=tau)
+  check_o(out, ref_o); check_score(s, ref_s)
+  # seeded mode: the oracle consumes the host twin of the in-kernel stream
+  es = oracle.seeded_exp_rand(77, B, H, S, S)
+  ref_o, ref_s = oracle.keyformer_forward(q, k, v, es, tau=tau)
+  out, s = ops.keyformer(qd, kd, vd, None, tau=tau, seed=77)
+  check_o(out, ref_o); check_score(s, ref_s)
+  # and the device materialisation of the stream equals the host twin
+  ed = ops.seeded_exp_rand(B, H, S, S, 77, gpu).cpu()
+  assert torch.allclose(ed, es, rtol=2e-6, atol=0)
+
+
+def test_rectangular_prefill_offset(gpu):
+  # Sq < Skv: query i sees keys j <= i + (Skv - Sq)  (cases/kernels/attn.py:23)
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 96, 2, 128, seed=3, kv_len=232)
+  ref_o, r1, r2 = oracle.roco_forward(q, k, v)
+  out, s1, s2 = ops.roco(qd, kd, vd)
+  check_o(out, ref_o); check_score(s1, r1); check_score(s2, r2)
+  er = oracle.prepare_exp_rand(1, 2, 96, 232, seed=3)
+  _, ref_kf = oracle.keyformer_forward(q, k, v, er, tau=1.5)
+  _, kf = ops.keyformer(qd, kd, vd, er.to(gpu), tau=1.5)
+  check_score(kf, ref_kf)
+  with pytest.raises(ValueError, match="Skv >= Sq"):
+    ops.attn(kd, qd, qd)
+
+
+def test_strided_views_and_bhsd_layout(gpu):
+  # [B,H,S,D] storage presented as a [B,S,H,D] view, and a q/k/v slice of a packed projection
+  B, S, H, D = 2, 160, 3, 128
+  (q, k, v), _ = gpu_inputs(gpu, B, S, H, D, seed=8)
+  qd = q.to(gpu).transpose(1, 2).contiguous().transpose(1, 2)
+  packed = torch.stack([q, k, v], dim=3).to(gpu)  # [B,S,H,3,D]
+  kd, vd = packed[:, :, :, 1], packed[:, :, :, 2]
+  assert not kd.is_contiguous() and not qd.is_contiguous()
+  ref_o, r1 = oracle.h2o_forward(q, k, v)
+  out, s1 = ops.h2o(qd, kd, vd)
+  check_o(out, ref_o); check_score(s1, r1)
+
+
+def test_bf16_inputs(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 192, 2, 128, seed=9, dtype=torch.bfloat16)
+  ref_o, r1 = oracle.h2o_forward(q, k, v)
+  out, s1 = ops.h2o(qd, kd, vd)
+  assert out.dtype == torch.bfloat16
+  check_o(out, ref_o, tight=2e-2)  # bf16 ulp at 1.0 is 7.8e-3
+  check_score(s1, r1)
+
+
+def test_fast_logits_mode_is_close(gpu):
+  # FT_FAST_LOGITS keeps QK^T/sqrt(D) in fp32: same O bar, looser scores (the fp16 rounding of the
+  # logits that the reference applies moves probabilities by ~1e-3)
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 256, 2, 128, seed=10)
+  ref_o, r1 = oracle.h2o_forward(q, k, v)
+  out, s1 = ops.h2o(qd, kd, vd, fast_logits=True)
+  check_o(out, ref_o); check_score(s1, r1, rel=2e-2)
+
+
+def test_non_causal(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 100, 2, 64, seed=11, kv_len=180)
+  qt, kt, vt = (t.transpose(1, 2).float() for t in (q, k, v))
+  s = (torch.matmul(q.transpose(1, 2), k.transpose(1, 2).transpose(-2, -1)) / np.sqrt(64)).float()
+  p = torch.softmax(s, -1)
+  ref_o = torch.matmul(p.half(), v.transpose(1, 2)).transpose(1, 2)
+  out, s1 = ops.h2o(qd, kd, vd, causal=False)
+  check_o(out, ref_o); check_score(s1, p.sum(2))
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "softmax_*.npz"))), ids=os.path.basename)
+def test_softmax_golden(gpu, path):
+  g = np.load(path, allow_pickle=False)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  _, (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  out, s1, s2 = ops.roco(qd, kd, vd)
+  check_o(out, torch.from_numpy(g["out"])); check_score(s1, torch.from_numpy(g["colsum"]))
+  check_score(s2, torch.from_numpy(g["colsumsq"]))
+  er = oracle.prepare_exp_rand(B, H, S, S, seed=seed).to(gpu)
+  check_score(ops.keyformer(qd, kd, vd, er, tau=1.5)[1], torch.from_numpy(g["kf_tensor_tau15"]))
+  check_score(ops.keyformer(qd, kd, vd, None, tau=1.0, seed=int(g["kf_seed"]))[1], torch.from_numpy(g["kf_seeded_tau1"]))
+  idx = ops.topk(s1, S // 8)
+  assert oracle.topk_agreement(idx.cpu(), torch.from_numpy(g["colsum"]), S // 8) == 0
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "linear_*.npz"))), ids=os.path.basename)
+def test_linear_golden(gpu, path):
+  g = np.load(path, allow_pickle=False)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  _, (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  check_o(ops.ea(qd, kd, vd), torch.from_numpy(g["ea"]))
+  check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), torch.from_numpy(g["sima"]))
+  check_sima(ops.sima(qd, kd, vd, normalize_q=False, out_dtype=torch.float32), torch.from_numpy(g["sima_rawq"]))
+
+
+def check_sima(out, ref, rel=1e-3):
+  """SimA outputs are ~1e-5 (fp16-subnormal range): compare in fp32 relative to the largest reference
+  magnitude; the fp16 output is checked against the fp16 rounding of the reference."""
+  out, ref = out.float().cpu(), ref.float()
+  assert torch.isfinite(out).all()
+  scale = ref.abs().max().item()
+  assert (out - ref).abs().max().item() <= rel * scale, f"sima {(out - ref).abs().max().item() / scale}"
+
+
+# ------------------------------------------------------------------ top-k heavy hitters
+
+def test_topk_matches_torch_and_orders_ties(gpu):
+  g = torch.Generator().manual_seed(0)
+  s = torch.randn(5, 7, 2048, generator=g).to(gpu)
+  idx = ops.topk(s, 256)
+  ref = torch.topk(s, 256, dim=-1).indices
+  assert idx.dtype == torch.int64 and torch.equal(idx, ref)
+  t = torch.tensor([[1.0, 3.0, 3.0, 0.5, 3.0, -1.0]], device=gpu)
+  assert ops.topk(t, 4).tolist() == [[1, 2, 4, 0]]  # ties: lower index first
+  s3 = torch.randn(3, 1000, generator=g).to(gpu)    # not a power of two
+  assert torch.equal(ops.topk(s3, 125), torch.topk(s3, 125).indices)
+
+
+# ------------------------------------------------------------------ builder / case modules
+
+def test_builder_callables_have_reference_signatures(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 128, 4, 128, seed=12)
+  f = ft.HipBuilder("attn", head_num=4, kv_head_num=4).build_callable()
+  out = f(qd, kd, vd)
+  assert isinstance(out, torch.Tensor) and out.shape == (1, 128, 4, 128) and out.device == qd.device
+  f = ft.HipBuilder("roco", head_num=4, kv_head_num=4).build_callable()
+  res = f(qd, kd, vd)
+  assert isinstance(res, tuple) and [t.shape for t in res] == [(1, 128, 4, 128), (1, 4, 128), (1, 4, 128)]
+  model = ft.get_model("kf", head_num=4, kv_head_num=4)
+  prep = model.prepare(batch_size=1, q_len=128, kv_len=128, device=gpu)
+  assert list(prep["input"]) == ["q", "k", "v", "exp_rand"] and prep["output"] == ["out", "kf_score"]
+  out, kf = model(*prep["input"].values())
+  ref_o, ref_kf = oracle.keyformer_forward(*(t.cpu() for t in prep["input"].values()), tau=1.5)
+  check_o(out, ref_o); check_score(kf, ref_kf)
+  h = ft.get_model("h2o", head_num=4, kv_head_num=4)
+  o, sc = h(qd, kd, vd)
+  assert h.heavy_hitters(sc).shape == (1, 4, 16)
+
+
+# ------------------------------------------------------------------ linear attention
+
+@pytest.mark.parametrize("B,S,H,seed", [(1, 128, 2, 0), (2, 200, 2, 1), (1, 1000, 3, 2), (1, 64, 1, 3), (1, 2500, 2, 4)])
+def test_ea_sima_small(gpu, B, S, H, seed):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, 64, seed=seed)
+  check_o(ops.ea(qd, kd, vd), oracle.ea_forward(q, k, v))
+  ref32 = oracle.sima_forward(q, k, v, out_dtype=torch.float32)
+  check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), ref32)
+  check_sima(ops.sima(qd, kd, vd, normalize_q=False, out_dtype=torch.float32),
+             oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32))
+  # fp16 output: within one fp16 (sub)normal step of the rounded fp32 reference
+  o16 = ops.sima(qd, kd, vd)
+  assert o16.dtype == torch.float16
+  assert (o16.float().cpu() - ref32.half().float()).abs().max().item() <= max(6e-8, 1e-3 * ref32.abs().max().item())
+
+
+def test_ea_sima_properties(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 512, 2, 64, seed=5)
+  c = torch.full_like(vd, 0.75)
+  assert (ops.ea(qd, kd, c).float() - 0.75).abs().max().item() < 2e-3         # weights sum to one on both sides
+  big = ops.ea(qd, kd * 30, vd)                                                # K up to ~120: exp must not overflow
+  assert torch.isfinite(big).all()
+  check_o(big, oracle.ea_forward(q, k * 30, v))
+  a = ops.sima(qd, kd, vd, out_dtype=torch.float32)
+  b = ops.sima(qd * 2, kd * 0.5, vd, out_dtype=torch.float32)                  # scale invariance of the L1 normalisation
+  assert torch.allclose(a, b, rtol=1e-4, atol=1e-9)
+
+
+# ------------------------------------------------------------------ the five measured configurations
+
+def test_config1_attn_b1_h32_s1024_d128(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 1024, 32, 128, seed=0)
+  check_o(ops.attn(qd, kd, vd), oracle.attn_forward(q, k, v))
+
+
+def test_config2_h2o_b1_h32_s2048_d128_with_topk(gpu):
+  S = 2048
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, 32, 128, seed=0)
+  ref_o, ref_s = oracle.chunked_over_heads(oracle.h2o_forward, (q, k, v), head_chunk=8)
+  out, s = ops.h2o(qd, kd, vd)
+  check_o(out, ref_o); check_score(s, ref_s)
+  idx = ops.topk(s, S // 8)
+  assert idx.shape == (1, 32, S // 8)
+  assert oracle.topk_agreement(idx.cpu(), ref_s, S // 8) == 0
+  assert torch.allclose(s.sum(-1).cpu(), torch.full((1, 32), float(S)), rtol=1e-4)
+
+
+def test_config3_keyformer_b1_h32_s4096_d128_tau1(gpu):
+  S, H, HS = 4096, 32, 2  # oracle on the first HS heads
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, 128, seed=0)
+  # seeded noise (the measured variant)
+  out, s = ops.keyformer(qd, kd, vd, None, tau=1.0, seed=2024)
+  es = oracle.seeded_exp_rand(2024, 1, HS, S, S)
+  ref_o, ref_s = oracle.keyformer_forward(q[:, :, :HS].contiguous(), k[:, :, :HS].contiguous(), v[:, :, :HS].contiguous(), es, tau=1.0)
+  check_o(out[:, :, :HS], ref_o); check_score(s[:, :HS], ref_s)
+  assert torch.allclose(s.sum(-1).cpu(), torch.full((1, H), float(S)), rtol=1e-4)
+  # tensor noise: degenerate noise E == 1 at tau == 1 must reproduce the H2O score on all heads
+  ones = torch.ones(1, H, S, S, dtype=torch.float32, device=gpu)
+  _, s_ones = ops.keyformer(qd, kd, vd, ones, tau=1.0)
+  _, s_h2o = ops.h2o(qd, kd, vd)
+  assert torch.allclose(s_ones, s_h2o, rtol=1e-5, atol=1e-7)
+  del ones
+  # tensor noise, reference recipe and default tau, oracle on the first heads
+  er = oracle.prepare_exp_rand(1, HS, S, S, seed=1)
+  big = torch.ones(1, H, S, S, dtype=torch.float32, device=gpu)
+  big[:, :HS] = er.to(gpu)
+  _, s_t = ops.keyformer(qd, kd, vd, big, tau=1.5)
+  _, ref_t = oracle.keyformer_forward(q[:, :, :HS].contiguous(), k[:, :, :HS].contiguous(), v[:, :, :HS].contiguous(), er, tau=1.5)
+  check_score(s_t[:, :HS], ref_t)
+
+
+def test_config4_roco_b4_h32_s4096_d128(gpu):
+  B, S, H = 4, 4096, 32
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, 128, seed=0)
+  out, s1, s2 = ops.roco(qd, kd, vd)
+  sl = (slice(3, 4), slice(None), slice(30, 32))  # last batch, last two heads
+  ref_o, r1, r2 = oracle.roco_forward(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous())
+  check_o(out[sl], ref_o); check_score(s1[3:4, 30:32], r1); check_score(s2[3:4, 30:32], r2)
+  assert torch.allclose(s1.sum(-1).cpu(), torch.full((B, H), float(S)), rtol=1e-4)
+  assert (s2 >= 0).all() and (s2 <= s1 * (1 + 1e-6)).all()
+  assert torch.equal(out[:, 0].cpu(), v[:, 0])
+  mean, var = ft.kernels.RoCo.mean_var(s1, s2, S)
+  assert (var > -1e-7).all() and torch.allclose(mean.sum(-1).cpu(), torch.ones(B, H), rtol=1e-4)
+  # q == 0: uniform causal rows => harmonic-number closed forms at full size
+  _, z1, z2 = ops.roco(torch.zeros_like(qd[:1, :, :2]), kd[:1, :, :2], vd[:1, :, :2])
+  inv = 1.0 / np.arange(1, S + 1)
+  assert np.abs(z1[0, 0].cpu().numpy() / np.cumsum(inv[::-1])[::-1] - 1).max() < 1e-4
+  assert np.abs(z2[0, 1].cpu().numpy() / np.cumsum((inv ** 2)[::-1])[::-1] - 1).max() < 1e-4
+
+
+def test_config5_ea_sima_b8_h16_s8192_d64(gpu):
+  B, S, H, D = 8, 8192, 16, 64
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=0)
+  check_o(ops.ea(qd, kd, vd), oracle.ea_forward(q, k, v))
+  check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), oracle.sima_forward(q, k, v, out_dtype=torch.float32))
+  o16 = ops.sima(qd, kd, vd)
+  ref16 = oracle.sima_forward(q, k, v)
+  assert (o16.float().cpu() - ref16.float()).abs().max().item() <= 1.2e-7  # two fp16 subnormal steps

@@ -1,0 +1,48 @@
+"""The CPU oracle against the committed golden vectors (tests/golden/*.npz, written by make_golden.py)."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _load(path):
+  z = np.load(path, allow_pickle=False)
+  return {k: z[k] for k in z.files}
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "softmax_*.npz"))), ids=os.path.basename)
+def test_softmax_cases_match_golden(path):
+  g = _load(path)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+  out, s1, s2 = oracle.roco_forward(q, k, v)
+  # thread count may change the reduction order of the CPU GEMM / sums by an ulp
+  assert np.abs(out.float().numpy() - g["out"].astype(np.float32)).max() <= 2e-3
+  np.testing.assert_allclose(s1.numpy(), g["colsum"], rtol=1e-5, atol=1e-7)
+  np.testing.assert_allclose(s2.numpy(), g["colsumsq"], rtol=1e-5, atol=1e-8)
+  _, kf = oracle.keyformer_forward(q, k, v, oracle.prepare_exp_rand(B, H, S, S, seed=seed), tau=1.5)
+  np.testing.assert_allclose(kf.numpy(), g["kf_tensor_tau15"], rtol=1e-5, atol=1e-7)
+  _, kfs = oracle.keyformer_forward(q, k, v, oracle.seeded_exp_rand(int(g["kf_seed"]), B, H, S, S), tau=1.0)
+  np.testing.assert_allclose(kfs.numpy(), g["kf_seeded_tau1"], rtol=1e-5, atol=1e-7)
+  assert oracle.topk_agreement(torch.from_numpy(g["topk"]), s1, S // 8) == 0
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "linear_*.npz"))), ids=os.path.basename)
+def test_linear_cases_match_golden(path):
+  g = _load(path)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+  assert np.abs(oracle.ea_forward(q, k, v).float().numpy() - g["ea"].astype(np.float32)).max() <= 1e-3
+  np.testing.assert_allclose(oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy(), g["sima"], rtol=1e-4, atol=1e-9)
+  np.testing.assert_allclose(oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32).numpy(),
+                             g["sima_rawq"], rtol=1e-4, atol=1e-7)
+
+
+def test_golden_files_present():
+  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 5
