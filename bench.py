@@ -1,0 +1,174 @@
+"""Benchmark of the fused attention + per-key score path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs]
+
+A step is one H2O call (attention forward + column-statistics pass, the two launches behind
+ft_attn_colstats_fwd) on B=1, H=32, S=4096, D=128 fp16 inputs already resident in HBM.  Prints ONE JSON
+line: whole-step throughput in algorithmic TFLOP/s (two causal S x S x D contractions, 2 B H S^2 D FLOP,
+whatever is recomputed internally), the roofline of the dominant kernel (the attention forward, timed
+with events on the launch stream), the CPU baseline (the oracle's eager restatement on the host cores,
+on a bounded subset of heads), and a per-configuration table for the five measured configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+# HBM bytes per launch of the attention kernel at the benchmark shape, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by a copy kernel of known size (profiles/attn_fwd_h2o_s4096_pmc.txt); None until measured
+ATTN_TRAFFIC_BYTES = None
+
+
+def event_time_us(fn, iters, warmup=3):
+  import torch
+  for _ in range(warmup):
+    fn()
+  start = torch.cuda.Event(enable_timing=True)
+  end = torch.cuda.Event(enable_timing=True)
+  torch.cuda.synchronize()
+  start.record()
+  for _ in range(iters):
+    fn()
+  end.record()
+  end.synchronize()
+  return start.elapsed_time(end) * 1e3 / iters
+
+
+def per_config_table(dev):
+  """µs per call, algorithmic TFLOP/s and GB/s with their roofline fractions for the five configurations."""
+  import torch
+  from flashtensor_amd import ops
+  rows = []
+
+  def qkv(B, S, H, D):
+    return tuple(torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3))
+
+  def add(name, shape, fn, flops, nbytes, iters=20):
+    us = event_time_us(fn, iters)
+    tf, gb = flops / us / 1e6, nbytes / us / 1e3
+    rows.append({"config": name, "shape": shape, "us": round(us, 1), "tflops": round(tf, 1),
+                 "mfma_frac": round(tf / PEAK_MFMA_TFLOPS, 4), "gbs": round(gb, 1), "hbm_frac": round(gb / PEAK_HBM_GBS, 4)})
+
+  def softmax_case(name, B, S, H, D, fn_of, extra_bytes=0):
+    q, k, v = qkv(B, S, H, D)
+    add(name, f"B{B} H{H} S{S} D{D}", fn_of(q, k, v), 2.0 * B * H * S * S * D, 4.0 * B * S * H * D * 2 + extra_bytes)
+
+  softmax_case("1 attn", 1, 1024, 32, 128, lambda q, k, v: (lambda: ops.attn(q, k, v)))
+  softmax_case("2 h2o+topk", 1, 2048, 32, 128,
+               lambda q, k, v: (lambda: ops.topk(ops.h2o(q, k, v)[1], 256)), extra_bytes=32 * 2048 * 4)
+  softmax_case("2' h2o", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.h2o(q, k, v)), extra_bytes=32 * 4096 * 4)
+  softmax_case("3 keyformer seeded tau=1", 1, 4096, 32, 128,
+               lambda q, k, v: (lambda: ops.keyformer(q, k, v, None, tau=1.0, seed=1)), extra_bytes=32 * 4096 * 4)
+  er = 1 + torch.randn(1, 32, 4096, 4096, dtype=torch.float32, device=dev).abs()
+  softmax_case("3t keyformer tensor noise tau=1.5", 1, 4096, 32, 128,
+               lambda q, k, v: (lambda: ops.keyformer(q, k, v, er, tau=1.5)), extra_bytes=2 * er.numel() * 4)
+  del er
+  softmax_case("4 roco", 4, 4096, 32, 128, lambda q, k, v: (lambda: ops.roco(q, k, v)), extra_bytes=2 * 4 * 32 * 4096 * 4)
+  q, k, v = qkv(8, 8192, 16, 64)
+  lin_flops, lin_bytes = 2 * 2.0 * 8 * 16 * 8192 * 64 * 64, 4.0 * 8 * 16 * 8192 * 64 * 2
+  add("5 ea", "B8 H16 S8192 D64", lambda: ops.ea(q, k, v), lin_flops, lin_bytes)
+  add("5 sima", "B8 H16 S8192 D64", lambda: ops.sima(q, k, v), lin_flops, lin_bytes)
+  return rows
+
+
+def cpu_baseline(B, S, H, D, heads):
+  """The oracle's eager H2O forward on `heads` of the H heads (heads are independent), host cores."""
+  import torch
+  import oracle
+  q, k, v = oracle.prepare_inputs(B, S, heads, D, seed=0)
+  oracle.h2o_forward(q[:, :256], k[:, :256], v[:, :256])  # warm the thread pool
+  t0 = time.perf_counter()
+  oracle.h2o_forward(q, k, v)
+  dt = time.perf_counter() - t0
+  flops = 2.0 * B * heads * S * S * D
+  return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+          "sample": f"oracle.h2o_forward on {heads} of {H} heads at S={S} (heads are independent), {dt:.2f} s wall",
+          "seconds": round(dt, 3), "host_cpus": os.cpu_count()}
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=50)
+  ap.add_argument("--warmup", type=int, default=10)
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+  ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
+  ap.add_argument("--cpu-heads", type=int, default=4)
+  args = ap.parse_args()
+  if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+    sys.exit("bench.py: this path runs on ONE GPU (heads/batches shard with no communication); run with --gpus 1")
+
+  import torch
+  from flashtensor_amd import _lib, ops
+  _lib.load()  # the HIP library is the only execution path
+  if not torch.cuda.is_available():
+    sys.exit("bench.py: no GPU visible")
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  torch.manual_seed(0)
+
+  B, H, S, D = 1, 32, 4096, 128
+  q, k, v = (torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3))
+  flops = 2.0 * B * H * S * S * D
+  alg_bytes = 4.0 * B * S * H * D * 2 + B * H * S * 4
+
+  def step():
+    return ops.h2o(q, k, v)
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  dt = (time.perf_counter() - t0) / args.steps
+
+  # dominant kernel: the attention forward with its normaliser output, events on the launch stream
+  attn_us = event_time_us(lambda: ops.attn(q, k, v, return_lse=True), max(10, args.steps))
+  step_us = event_time_us(step, max(10, args.steps))
+  attn_tflops = flops / attn_us / 1e6
+
+  result = {
+      "metric": "fused attn+score (H2O) algorithmic TFLOP/s at S=4096, 1 GPU",
+      "value": round(flops / dt / 1e12, 2),
+      "unit": "TFLOP/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": round(dt * 1e3, 5),
+      "us_per_step": round(dt * 1e6, 1),
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "f16",
+      "data": "synthetic",
+      "config": {"workload": "H2O fused attention + per-key column sums, causal, B=1 H=32 S=4096 D=128 fp16",
+                 "launches_per_step": ["attn_fwd_kernel", "colstats_kernel"], "logits": "reference fp16 rounding"},
+      "frac_of_fp16_mfma_peak": round(flops / dt / 1e12 / PEAK_MFMA_TFLOPS, 4),
+      "algorithmic_gbs": round(alg_bytes / dt / 1e9, 1),
+      "roofline": {"bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(attn_tflops, 1), "peak": PEAK_MFMA_TFLOPS,
+                   "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_MFMA_TFLOPS, 4), "traffic": ATTN_TRAFFIC_BYTES,
+                   "us_per_launch": round(attn_us, 1), "algorithmic_flop_per_launch": flops},
+      "kernels_us": {"attn_fwd_kernel": round(attn_us, 1), "colstats_kernel": round(step_us - attn_us, 1),
+                     "step_events": round(step_us, 1)},
+  }
+  if not args.no_configs:
+    result["per_config"] = per_config_table(dev)
+  if not args.no_cpu:
+    result["cpu_baseline"] = cpu_baseline(B, S, H, D, args.cpu_heads)
+  else:
+    result["cpu_baseline"] = None
+  print(json.dumps(result))
+
+
+if __name__ == "__main__":
+  main()
