@@ -19,6 +19,7 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 #define FT_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
@@ -61,6 +62,13 @@ __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane
 
 // Value held by the partner lane l ^ 32 (the other 16 rows of a 32x32 accumulator column).
 __device__ __forceinline__ float xchg32(float x) { return __shfl_xor(x, 32); }
+
+// max of three without the NaN-quieting moves the compiler adds around fmaxf on MFMA results
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
@@ -109,6 +117,44 @@ __device__ __forceinline__ void stage_tile(const uint16_t* __restrict__ src, int
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, FT_LDS(void, dst), 16, 0, 0);
   }
 }
+
+// The same copy with the per-lane source offsets computed once: tiles of one operand differ only by a
+// wave-uniform base address, so a full tile costs one direct-to-LDS load per round and no address
+// arithmetic.  Offsets are 32-bit byte offsets from row 0 of the tile (hosts check they fit).
+template <int D, int ROWS, int NT, int SWZ>
+struct TileStager {
+  typedef TileGeom<D> G;
+  static constexpr int ROUNDS = ROWS * G::CPR / NT;
+  uint32_t off[ROUNDS];
+
+  __device__ __forceinline__ void init(int64_t row_stride) {
+    const int lane = lane_id();
+    const int wave = wave_id();
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) {
+      const int slot = it * NT + wave * 64 + lane;
+      const int r = slot / G::CPR;
+      const int cs = slot % G::CPR;
+      const int c = cs ^ (SWZ == kRowSwizzle ? G::row_swz(r) : G::tr_swz(r));
+      off[it] = (uint32_t)((r * row_stride + c * 8) * 2);
+    }
+  }
+
+  // `src` (row 0 of the tile) must be wave-uniform.
+  __device__ __forceinline__ void issue(const uint16_t* src, int64_t row_stride, int rows_valid, char* lds_tile) const {
+    if (rows_valid >= ROWS) {
+      const int wave = wave_id();
+      const char* base = reinterpret_cast<const char*>(src);
+#pragma unroll
+      for (int it = 0; it < ROUNDS; ++it) {
+        char* dst = lds_tile + (it * NT + wave * 64) * 16;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off[it]), FT_LDS(void, dst), 16, 0, 0);
+      }
+    } else {
+      stage_tile<D, ROWS, NT, SWZ>(src, row_stride, rows_valid, lds_tile);
+    }
+  }
+};
 
 // 8 contiguous elements (one 16-byte chunk `c`) of row `r` from a kRowSwizzle tile.
 template <int D, typename V8>
