@@ -121,6 +121,10 @@ int validate_attn(const FtAttnArgs* a, bool need_v_o) {
     return fail(FT_EINVAL, "q, k, v, o must be 16-byte aligned");
   if (!stride_ok(a->sq) || !stride_ok(a->sk) || (need_v_o && (!stride_ok(a->sv) || !stride_ok(a->so))))
     return fail(FT_EINVAL, "strides must be positive multiples of 8 elements with a contiguous head_dim axis");
+  // tiles are fetched with 32-bit byte offsets from the (b, h) base of each operand
+  if ((int64_t)a->Sq * a->sq.s * 2 >= 0x7fffffffLL || (int64_t)a->Skv * a->sk.s * 2 >= 0x7fffffffLL ||
+      (need_v_o && (int64_t)a->Skv * a->sv.s * 2 >= 0x7fffffffLL))
+    return fail(FT_EUNSUPPORTED, "sequence stride too large: S * stride_s must stay below 2^30 elements");
   const int64_t wgs = (int64_t)a->B * a->H * (((int64_t)(a->Sq > a->Skv ? a->Sq : a->Skv) + 63) / 64);
   if (wgs > 0x7fffffffLL) return fail(FT_EUNSUPPORTED, "problem too large for one launch");
   return FT_OK;
@@ -287,6 +291,8 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
     return fail(FT_EINVAL, "q, k, v, o must be 16-byte aligned");
   if (!stride_ok(a->sq) || !stride_ok(a->sk) || !stride_ok(a->sv) || !stride_ok(a->so))
     return fail(FT_EINVAL, "strides must be positive multiples of 8 elements with a contiguous head_dim axis");
+  if ((int64_t)a->Sq * a->sk.s * 2 >= 0x7fffffffLL || (int64_t)a->Sq * a->sv.s * 2 >= 0x7fffffffLL)
+    return fail(FT_EUNSUPPORTED, "sequence stride too large: S * stride_s must stay below 2^30 elements");
   const size_t need = ft::linattn_workspace_bytes(*a, kind);
   if (!workspace || workspace_bytes < need)
     return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);

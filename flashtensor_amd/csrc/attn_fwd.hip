@@ -40,6 +40,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   typedef typename T::vec8 vec8;
   constexpr int TILE_BYTES = BN * G::RB;
   constexpr bool kIsF16 = __is_same(typename T::elem, _Float16);
+  constexpr bool kFastMasked = kIsF16 && EMU && KF == kKfNone;  // variants served by the packed-fp16 softmax
   // Software pipeline across tiles: the QK^T MFMAs of tile it+1 are issued in the same iteration as the
   // softmax (VALU) and PV MFMAs of tile it, so the matrix and vector pipes overlap inside one wave.
   // K therefore runs one tile ahead of V in LDS.
@@ -95,13 +96,13 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
 
   TileStager<D, BN, NT, kRowSwizzle> stK;
   TileStager<D, BN, NT, kTrSwizzle> stV;
-  stK.init(p.sk.s);
-  stV.init(p.sv.s);
+  stK.init(kbase, p.sk.s);
+  stV.init(vbase, p.sv.s);
   auto stage_k = [&](int t, char* dst) {
-    if (t < ntiles) stK.issue(kbase + (int64_t)t * BN * p.sk.s, p.sk.s, min(BN, p.Skv - t * BN), dst);
+    if (t < ntiles) stK.issue(t * BN, min(BN, p.Skv - t * BN), dst);
   };
   auto stage_v = [&](int t, char* dst) {
-    if (t < ntiles) stV.issue(vbase + (int64_t)t * BN * p.sv.s, p.sv.s, min(BN, p.Skv - t * BN), dst);
+    if (t < ntiles) stV.issue(t * BN, min(BN, p.Skv - t * BN), dst);
     if (KF == kKfSeeded && t < ntiles && threadIdx.x < BN)
       ldsCol[(t & 1) * BN + threadIdx.x] = noise_col(nk, (uint32_t)(t * BN + threadIdx.x));
   };
@@ -115,24 +116,56 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   float m_kf = NEG_INF, l_kf = 0.f;
   float16v S0[2], S1[2];  // score accumulators of the current / next tile (they swap every tile)
 
-  // ---- S^T = K Q^T : [64 keys] x [32 queries] as two 32x32 blocks, operand reads one step ahead
-  auto qk = [&](float16v (&s)[2], const char* tk) {
+  // Per-lane LDS byte offsets of the MFMA operand reads inside a tile (the XOR swizzles make them
+  // lane-dependent, so they are computed once instead of per read).
+  uint32_t koff[KSTEPS];  // K row n (and n + 32 via an immediate), chunk 2t + g
 #pragma unroll
-    for (int mbk = 0; mbk < 2; ++mbk)
+  for (int t = 0; t < KSTEPS; ++t) koff[t] = n * G::RB + (((2 * t + g) ^ G::row_swz(n)) << 4);
+  uint32_t voff[DB];  // V^T operand: rows 4g + (l%16)/4 (+ 16 ks, + 8 via immediates), columns 32 db + ...
+  {
+    const int j16 = lane & 15, dhalf = (lane >> 4) & 1;
+    const int r0 = 4 * g + (j16 >> 2);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[mbk][r] = 0.f;
-    vec8 ka[2][2];
-#pragma unroll
-    for (int mbk = 0; mbk < 2; ++mbk) ka[0][mbk] = read_row_chunk<D, vec8>(tk, mbk * 32 + n, g);
-#pragma unroll
-    for (int t = 0; t < KSTEPS; ++t) {
-      if (t + 1 < KSTEPS) {
-#pragma unroll
-        for (int mbk = 0; mbk < 2; ++mbk) ka[(t + 1) & 1][mbk] = read_row_chunk<D, vec8>(tk, mbk * 32 + n, 2 * (t + 1) + g);
-      }
-#pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk) s[mbk] = T::mfma(ka[t & 1][mbk], qf[t], s[mbk]);
+    for (int db = 0; db < DB; ++db) {
+      const int d0 = 32 * db + 16 * dhalf + 4 * (j16 & 3);
+      voff[db] = r0 * G::RB + (((d0 >> 3) ^ G::tr_swz(r0)) << 4) + (d0 & 7) * 2;
     }
+  }
+
+  // ---- S^T = K Q^T : [64 keys] x [32 queries] as two 32x32 blocks (16 LDS reads, 16 MFMAs), optionally
+  // in two halves over the head dimension so that other work can sit between them
+  auto qk_part = [&](float16v (&s)[2], const char* tk, auto t0_tag, auto t1_tag) {
+    constexpr int T0 = decltype(t0_tag)::value, T1 = decltype(t1_tag)::value;
+    if (T0 == 0) {
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[mbk][r] = 0.f;
+    }
+    vec8 ka[KSTEPS][2];
+#pragma unroll
+    for (int t = T0; t < T1; ++t)
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) ka[t][mbk] = *reinterpret_cast<const vec8*>(tk + koff[t] + mbk * 32 * G::RB);
+#pragma unroll
+    for (int t = T0; t < T1; ++t)
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) s[mbk] = T::mfma(ka[t][mbk], qf[t], s[mbk]);
+  };
+  auto qk = [&](float16v (&s)[2], const char* tk) {
+    qk_part(s, tk, std::integral_constant<int, 0>{}, std::integral_constant<int, KSTEPS>{});
+  };
+  // LDS latency is far longer than an MFMA, so operand reads must run several MFMAs ahead of their
+  // consumers; sched_group_barrier sequences pin that order (the scheduler would otherwise sink each
+  // read next to its use to save registers).  Masks: 0x008 MFMA, 0x100 LDS read, 0x002 VALU.
+  auto sched_qk_alone = [&]() {
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int t = 0; t < KSTEPS - 3; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
   };
 
   auto rescale = [&](float rowmax) {
@@ -149,41 +182,78 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     }
   };
 
+  // ---- mask-free fp16 softmax, in two parts so that the rescale branch sits between them.
+  // Rounding is monotonic, so the row maximum of the rounded logits is the rounded maximum of the raw
+  // accumulators.
+  auto fast_max = [&](const float16v (&s)[2]) {
+    // four independent chains, then a short tree: the reduction is latency-, not throughput-bound
+    float m4[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int mbk = c >> 1, r0 = (c & 1) * 8;
+      m4[c] = max3(s[mbk][r0], s[mbk][r0 + 1], s[mbk][r0 + 2]);
+      m4[c] = max3(m4[c], s[mbk][r0 + 3], s[mbk][r0 + 4]);
+      m4[c] = max3(m4[c], s[mbk][r0 + 5], s[mbk][r0 + 6]);
+      m4[c] = __builtin_fmaxf(m4[c], s[mbk][r0 + 7]);
+    }
+    float amax = __builtin_fmaxf(max3(m4[0], m4[1], m4[2]), m4[3]);
+    amax = __builtin_fmaxf(amax, xchg32(amax));
+    rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
+  };
+  // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.  The row
+  // maximum above is taken over hidden keys too: any upper bound of the visible logits is a valid
+  // stabiliser, and hidden logits come from the same distribution.
+  auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const float neg_m = -m_run;
+    const half2v ones = {(_Float16)1.f, (_Float16)1.f};
+    // local key index of register r is 32 mbk + 8 (r / 4) + 4 g + r % 4; it is visible iff <= lim + 4 g
+    const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0 - 4 * g;
+    uint4v pw[4];
+    // Eight elements (one MFMA operand) at a time, stage by stage, so that consecutive instructions are
+    // independent: every stage's result is needed only four instructions later.
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      const int mbk = blk >> 1, rb = (blk & 1) * 8;
+      half2v h2[4];
+      _Float16 t[8];
+      float x[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float2v a2 = {s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]};
+        h2[i] = __builtin_convertvector(a2, half2v);  // QK^T is an fp16 tensor in the reference
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) t[i] = (_Float16)((float)h2[i >> 1][i & 1] * p.logit_mul);  // ... divided by sqrt(D) in fp16
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x[i] = __builtin_fmaf((float)t[i], kLog2e, neg_m);
+        if (MASKED) {
+          const int jl = 32 * mbk + 8 * ((rb + i) >> 2) + ((rb + i) & 3);
+          x[i] = (jl > lim) ? NEG_INF : x[i];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = __builtin_amdgcn_exp2f(x[i]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float2v p2 = {x[2 * i], x[2 * i + 1]};
+        const half2v ph = __builtin_convertvector(p2, half2v);
+        l_run = __builtin_amdgcn_fdot2(ph, ones, l_run, false);  // row sum of the fp16 P the MFMA consumes
+        pw[blk][i] = __builtin_bit_cast(uint32_t, ph);           // whole 32-bit words: no 16-bit shuffles
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
+  };
+
   // ---- softmax of one tile: s (raw accumulators) -> pb (16-bit unnormalised probabilities)
   auto softmax = [&](auto masked_tag, float16v (&s)[2], vec8 (&pb)[4], int n0, int buf, const float (&er)[2][16]) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    if constexpr (kIsF16 && EMU && !MASKED && KF == kKfNone) {
-      // Fast path.  Rounding is monotonic, so the row maximum of the rounded logits is the rounded
-      // maximum of the raw accumulators.
-      float amax = max3(s[0][0], s[0][1], s[1][0]);
-#pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) amax = max3(amax, s[mbk][r], s[mbk][r + 1]);
-      amax = fmaxf(amax, xchg32(amax));
-      rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
-      const float neg_m = -m_run;
-      const half2v ones = {(_Float16)1.f, (_Float16)1.f};
-      uint4v pw[4];
-#pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float2v a2 = {s[mbk][r], s[mbk][r + 1]};
-          const half2v h2 = __builtin_convertvector(a2, half2v);       // QK^T is an fp16 tensor in the reference
-          const _Float16 t0 = (_Float16)((float)h2[0] * p.logit_mul);  // ... divided by sqrt(D) in fp16
-          const _Float16 t1 = (_Float16)((float)h2[1] * p.logit_mul);
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf((float)t0, kLog2e, neg_m));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf((float)t1, kLog2e, neg_m));
-          const float2v p2 = {p0, p1};
-          const half2v ph = __builtin_convertvector(p2, half2v);
-          l_run = __builtin_amdgcn_fdot2(ph, ones, l_run, false);  // row sum of the fp16 P the MFMA consumes
-          pw[2 * mbk + (r >> 3)][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);  // whole 32-bit words: no 16-bit shuffles
-        }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
+    if constexpr (false) {
     } else {
       // ---- logits in the log2 domain, with the reference's rounding points when EMU
+      const int jmax = CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1;  // last key this query sees
       float rowmax = NEG_INF;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk)
@@ -199,7 +269,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
           }
           if (MASKED) {
             const int j = n0 + 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
-            if ((CAUSAL && j > qi + p.off) || j >= p.Skv) x = NEG_INF;
+            x = (j > jmax) ? NEG_INF : x;
           }
           s[mbk][r] = x;
           rowmax = fmaxf(rowmax, x);
@@ -253,19 +323,68 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     }
   };
 
-  // ---- O^T += V^T P^T (operand reads one step ahead of the MFMAs)
+  // ---- O^T += V^T P^T (32 transposed LDS reads, 16 MFMAs)
+  auto read_vt = [&](const char* tv, int ks, int db) -> vec8 {
+    const char* p0 = tv + voff[db] + ks * 16 * G::RB;
+    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(FT_LDS(short4v, p0));
+    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(FT_LDS(short4v, p0 + 8 * G::RB));
+    short8v both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, both);
+  };
   auto pv = [&](const vec8 (&pb)[4], const char* tv) {
-    vec8 va[2][DB];
+    vec8 va[4][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) va[0][db] = read_tr_operand<D, vec8>(tv, 0, 32 * db);
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      if (ks + 1 < 4) {
+      for (int db = 0; db < DB; ++db) va[ks][db] = read_vt(tv, ks, db);
 #pragma unroll
-        for (int db = 0; db < DB; ++db) va[(ks + 1) & 1][db] = read_tr_operand<D, vec8>(tv, 16 * (ks + 1), 32 * db);
-      }
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma(va[ks & 1][db], pb[ks], o_acc[db]);
+      for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma(va[ks][db], pb[ks], o_acc[db]);
+  };
+  auto sched_pv_alone = [&]() {
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
+#pragma unroll
+    for (int i = 0; i < 4 * DB - 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
+  };
+
+  // One tile of the pipelined loop (fp16, reference rounding): the QK^T MFMAs of the next tile and the PV
+  // MFMAs of this tile are spread over this tile's softmax VALU instructions (only about four hide
+  // behind one MFMA, so the two kinds are interleaved as finely as the dependencies allow).  The first
+  // half of QK^T covers the latency of the row-maximum reduction and of the (rare) rescale branch.
+  auto fast_tile = [&](auto masked_tag, auto stage_tag, float16v (&s_cur)[2], float16v (&s_next)[2], const char* tk_next,
+                       const char* tv, int n0, int it, char* k_dst, char* v_dst) {
+    constexpr bool STAGE = decltype(stage_tag)::value;
+    vec8 pb[4];
+    // STAGE: the direct-to-LDS loads of K[it+2] and V[it+1] (both full tiles) are issued from inside this
+    // block, one every few MFMAs.  Issued back to back they fill the texture-address queue (one 1 KB load
+    // per 16 cycles per CU) and the wave stalls at issue for about a sixth of the tile time.
+    qk_part(s_next, tk_next, std::integral_constant<int, 0>{}, std::integral_constant<int, KSTEPS / 2>{});
+    fast_max(s_cur);
+    if (STAGE) {  // after the rescale branch, so that the loads share a basic block with most of the MFMAs
+      stK.issue_full((it + 2) * BN, k_dst);
+      stV.issue_full((it + 1) * BN, v_dst);
+    }
+    qk_part(s_next, tk_next, std::integral_constant<int, KSTEPS / 2>{}, std::integral_constant<int, KSTEPS>{});
+    fast_exp(masked_tag, s_cur, pb, n0);
+    pv(pb, tv);
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 2);
+#pragma unroll
+    for (int i = 0; i < KSTEPS; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 2);
+    }
+#pragma unroll
+    for (int i = 0; i < 4 * DB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
+      if (STAGE && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 2);
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 2);
     }
   };
 
@@ -305,29 +424,36 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   wait_vmem();
   __syncthreads();
   qk(S0, ldsK0);
+  sched_qk_alone();
 
   int it = 0;
   // ---- mask-free tiles, two per trip so that the two score buffers swap roles without copies
-  const int nf2 = n_fast & ~1;
+  // pairs (it, it+1) of mask-free tiles whose staged tiles K[it+2], K[it+3], V[it+1], V[it+2] are whole tiles
+  const int nf2 = max(0, min(n_fast, p.Skv / BN - 2)) & ~1;
   for (; it < nf2; it += 2) {
-    vec8 pb[4];
-    sync_and_stage(it, true, ldsK0, ldsV1);      // K[it+2], V[it+1]
-    qk(S1, ldsK1);                               // tile it+1
-    softmax(std::false_type{}, S0, pb, it * BN, 0, er);
-    pv(pb, ldsV0);
-    sync_and_stage(it + 1, true, ldsK1, ldsV0);  // K[it+3], V[it+2]
-    qk(S0, ldsK0);  // tile it+2; past the last tile this reads stale LDS and is discarded
-    softmax(std::false_type{}, S1, pb, (it + 1) * BN, 1, er);
-    pv(pb, ldsV1);
+    wait_vmem();
+    __syncthreads();
+    fast_tile(std::false_type{}, std::true_type{}, S0, S1, ldsK1, ldsV0, 0, it, ldsK0, ldsV1);      // stages K[it+2], V[it+1]
+    wait_vmem();
+    __syncthreads();
+    fast_tile(std::false_type{}, std::true_type{}, S1, S0, ldsK0, ldsV1, 0, it + 1, ldsK1, ldsV0);  // stages K[it+3], V[it+2]
   }
-  // ---- tiles that straddle the diagonal or the end of K (and every tile of the KeyFormer variants)
+  // ---- tiles that straddle the diagonal or the end of K (and every tile of the other variants)
   for (; it < nw; ++it) {
-    vec8 pb[4];
     const bool odd = it & 1;
     sync_and_stage(it, true, odd ? ldsK1 : ldsK0, odd ? ldsV0 : ldsV1);
-    softmax(std::true_type{}, S0, pb, it * BN, it & 1, er);
-    pv(pb, odd ? ldsV1 : ldsV0);
-    qk(S0, odd ? ldsK0 : ldsK1);
+    if constexpr (kFastMasked) {
+      fast_tile(std::true_type{}, std::false_type{}, S0, S1, odd ? ldsK0 : ldsK1, odd ? ldsV1 : ldsV0, it * BN, it, nullptr, nullptr);
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) S0[mbk] = S1[mbk];
+    } else {
+      vec8 pb[4];
+      softmax(std::true_type{}, S0, pb, it * BN, it & 1, er);
+      pv(pb, odd ? ldsV1 : ldsV0);
+      sched_pv_alone();
+      qk(S0, odd ? ldsK0 : ldsK1);
+      sched_qk_alone();
+    }
   }
   // ---- tiles entirely above this wave's diagonal: keep the workgroup's barriers and staging in step
   for (; it < ntiles; ++it) sync_and_stage(it, false, (it & 1) ? ldsK1 : ldsK0, (it & 1) ? ldsV0 : ldsV1);
@@ -363,10 +489,9 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
 
 template <typename T, int D, bool CAUSAL, bool EMU, int KF>
 static hipError_t launch_one(const AttnKernelParams& p, hipStream_t stream) {
-  auto kern = attn_fwd_kernel<T, D, CAUSAL, EMU, KF>;
   const int nMB = (p.Sq + kAttnBM - 1) / kAttnBM;
   dim3 grid((unsigned)(nMB * p.B * p.H));
-  hipLaunchKernelGGL(kern, grid, dim3(kAttnThreads), 0, stream, p);
+  hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF>), grid, dim3(kAttnThreads), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -75,9 +75,11 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
   if (MODE == kStatKfTensor) er_col = p.exp_rand + b * p.er_sb + h * p.er_sh + kj_c;
 
   float sum = 0.f, sumsq = 0.f;
+  TileStager<D, BQ, NT, kRowSwizzle> stQ;
+  stQ.init(qbase, p.sq.s);
 
   if (ntiles > 0) {
-    stage_tile<D, BQ, NT, kRowSwizzle>(qbase + (int64_t)i_begin * p.sq.s, p.sq.s, min(BQ, p.Sq - i_begin), ldsQ);
+    stQ.issue(i_begin, min(BQ, p.Sq - i_begin), ldsQ);
     if (threadIdx.x < BQ) {
       const int i = i_begin + threadIdx.x;
       ldsLse[threadIdx.x] = i < p.Sq ? lse_bh[i] : POS_INF;
@@ -112,8 +114,7 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
 
     if (has_next) {
       const int in = i0 + BQ;
-      stage_tile<D, BQ, NT, kRowSwizzle>(qbase + (int64_t)in * p.sq.s, p.sq.s, min(BQ, p.Sq - in),
-                                         ldsQ + (buf ^ 1) * TILE_BYTES);
+      stQ.issue(in, min(BQ, p.Sq - in), ldsQ + (buf ^ 1) * TILE_BYTES);
     }
 
     const int wave_key0 = j0 + wave * 32;

@@ -61,7 +61,19 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
 
 // Value held by the partner lane l ^ 32 (the other 16 rows of a 32x32 accumulator column).
-__device__ __forceinline__ float xchg32(float x) { return __shfl_xor(x, 32); }
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second:
+// called with (x, x) it returns {x[0..31], x[0..31]} and {x[32..63], x[32..63]}; every lane then holds
+// both values of its pair.  One VALU instruction instead of an LDS round trip.
+__device__ __forceinline__ float xchg32(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t lo = r[0], hi = r[1];
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? lo : hi);
+#else
+  return x;
+#endif
+}
 
 // max of three without the NaN-quieting moves the compiler adds around fmaxf on MFMA results
 __device__ __forceinline__ float max3(float a, float b, float c) {
@@ -92,42 +104,41 @@ struct TileGeom {
 
 enum Swizzle { kRowSwizzle = 0, kTrSwizzle = 1 };
 
-// Cooperative global -> LDS copy of a ROWS x D tile by NT threads with direct-to-LDS loads
-// (global_load_lds_dwordx4: LDS address = wave-uniform base + lane * 16).  The swizzle is applied on
-// the global side: the lane that fills LDS slot (r, c') fetches global chunk c' ^ swz(r).
-// `src` points at row 0 of the tile, `row_stride` in elements; rows >= rows_valid re-read the last valid
-// row (callers mask them).  Completion: wait_vmem() then a workgroup barrier.
-template <int D, int ROWS, int NT, int SWZ>
-__device__ __forceinline__ void stage_tile(const uint16_t* __restrict__ src, int64_t row_stride, int rows_valid,
-                                           char* lds_tile) {
-  typedef TileGeom<D> G;
-  constexpr int CHUNKS = ROWS * G::CPR;
-  static_assert(CHUNKS % NT == 0, "tile must be a whole number of rounds");
-  const int lane = lane_id();
-  const int wave = wave_id();
-#pragma unroll
-  for (int it = 0; it < CHUNKS / NT; ++it) {
-    const int slot = it * NT + wave * 64 + lane;  // 16-byte slot index in the tile
-    const int r = slot / G::CPR;
-    const int cs = slot % G::CPR;
-    const int c = cs ^ (SWZ == kRowSwizzle ? G::row_swz(r) : G::tr_swz(r));
-    const int rr = r < rows_valid ? r : rows_valid - 1;
-    const uint16_t* g = src + (int64_t)rr * row_stride + c * 8;
-    char* dst = lds_tile + (it * NT + wave * 64) * 16;  // wave-uniform
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, FT_LDS(void, dst), 16, 0, 0);
-  }
+// Cooperative global -> LDS copy of ROWS x D tiles by NT threads with direct-to-LDS buffer loads
+// (buffer_load_dwordx4 ... lds: LDS address = wave-uniform base + lane * 16; the MUBUF form, unlike the
+// global_load form, does not make the compiler treat every later LDS wait as a full drain).  The swizzle
+// is applied on the global side: the lane that fills LDS slot (r, c') fetches global chunk c' ^ swz(r).
+// Per-lane byte offsets are computed once; a tile then costs one load per round with a scalar tile offset.
+// Rows >= rows_valid re-read the last valid row (callers mask them).  Completion: wait_vmem() then a
+// workgroup barrier.  All byte offsets from `base` must fit in 31 bits (checked by the host).
+// The host pass only parses kernel bodies (to emit launch stubs); the buffer-resource type and builtins
+// exist in the device pass only.
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
 }
+__device__ __forceinline__ void load_lds16(rsrc_t rsrc, char* lds_dst, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, FT_LDS(void, lds_dst), 16, voff, soff, 0, 0);
+}
+#else
+typedef int rsrc_t;
+__device__ inline rsrc_t make_rsrc(const void*) { return 0; }
+__device__ inline void load_lds16(rsrc_t, char*, uint32_t, uint32_t) {}
+#endif
 
-// The same copy with the per-lane source offsets computed once: tiles of one operand differ only by a
-// wave-uniform base address, so a full tile costs one direct-to-LDS load per round and no address
-// arithmetic.  Offsets are 32-bit byte offsets from row 0 of the tile (hosts check they fit).
 template <int D, int ROWS, int NT, int SWZ>
 struct TileStager {
   typedef TileGeom<D> G;
   static constexpr int ROUNDS = ROWS * G::CPR / NT;
+  static_assert((ROWS * G::CPR) % NT == 0, "tile must be a whole number of rounds");
+  rsrc_t rsrc;
   uint32_t off[ROUNDS];
+  uint32_t row_bytes;
 
-  __device__ __forceinline__ void init(int64_t row_stride) {
+  __device__ __forceinline__ void init(const uint16_t* base, int64_t row_stride) {
+    rsrc = make_rsrc(base);
+    row_bytes = (uint32_t)(row_stride * 2);
     const int lane = lane_id();
     const int wave = wave_id();
 #pragma unroll
@@ -136,22 +147,40 @@ struct TileStager {
       const int r = slot / G::CPR;
       const int cs = slot % G::CPR;
       const int c = cs ^ (SWZ == kRowSwizzle ? G::row_swz(r) : G::tr_swz(r));
-      off[it] = (uint32_t)((r * row_stride + c * 8) * 2);
+      off[it] = (uint32_t)r * row_bytes + c * 16;
     }
   }
 
-  // `src` (row 0 of the tile) must be wave-uniform.
-  __device__ __forceinline__ void issue(const uint16_t* src, int64_t row_stride, int rows_valid, char* lds_tile) const {
+  // A tile known to lie entirely inside the operand: straight-line code (one load per round) that a
+  // caller can spread between other instructions.
+  __device__ __forceinline__ void issue_full(int row0, char* lds_tile) const {
+    const int wave = wave_id();
+    const uint32_t tile_off = (uint32_t)row0 * row_bytes;  // wave-uniform
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) {
+      char* dst = lds_tile + (it * NT + wave * 64) * 16;
+      load_lds16(rsrc, dst, off[it], tile_off);
+    }
+  }
+
+  // Tile whose row 0 is row `row0` of the operand.
+  __device__ __forceinline__ void issue(int row0, int rows_valid, char* lds_tile) const {
+    const int wave = wave_id();
+    const uint32_t tile_off = (uint32_t)row0 * row_bytes;  // wave-uniform
     if (rows_valid >= ROWS) {
-      const int wave = wave_id();
-      const char* base = reinterpret_cast<const char*>(src);
+      issue_full(row0, lds_tile);
+    } else {
+      const int lane = lane_id();
 #pragma unroll
       for (int it = 0; it < ROUNDS; ++it) {
+        const int slot = it * NT + wave * 64 + lane;
+        const int r = slot / G::CPR;
+        const int cs = slot % G::CPR;
+        const int c = cs ^ (SWZ == kRowSwizzle ? G::row_swz(r) : G::tr_swz(r));
+        const int rr = r < rows_valid ? r : rows_valid - 1;
         char* dst = lds_tile + (it * NT + wave * 64) * 16;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off[it]), FT_LDS(void, dst), 16, 0, 0);
+        load_lds16(rsrc, dst, (uint32_t)rr * row_bytes + c * 16, tile_off);
       }
-    } else {
-      stage_tile<D, ROWS, NT, SWZ>(src, row_stride, rows_valid, lds_tile);
     }
   }
 };

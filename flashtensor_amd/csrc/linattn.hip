@@ -104,8 +104,11 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 #pragma unroll
   for (int e = 0; e < 8; ++e) qabs[e] = 0.f;
 
-  stage_tile<D, TILE, NT, kTrSwizzle>(kbase + (int64_t)tok_begin * p.sk.s, p.sk.s, min(TILE, p.S - tok_begin), ldsK);
-  stage_tile<D, TILE, NT, kTrSwizzle>(vbase + (int64_t)tok_begin * p.sv.s, p.sv.s, min(TILE, p.S - tok_begin), ldsV);
+  TileStager<D, TILE, NT, kTrSwizzle> stK, stV;
+  stK.init(kbase, p.sk.s);
+  stV.init(vbase, p.sv.s);
+  stK.issue(tok_begin, min(TILE, p.S - tok_begin), ldsK);
+  stV.issue(tok_begin, min(TILE, p.S - tok_begin), ldsV);
 
   for (int it = 0; it < ntiles; ++it) {
     const int t0 = tok_begin + it * TILE;
@@ -129,8 +132,8 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 
     if (it + 1 < ntiles) {
       const int tn = t0 + TILE;
-      stage_tile<D, TILE, NT, kTrSwizzle>(kbase + (int64_t)tn * p.sk.s, p.sk.s, min(TILE, p.S - tn), ldsK + (buf ^ 1) * TILE_BYTES);
-      stage_tile<D, TILE, NT, kTrSwizzle>(vbase + (int64_t)tn * p.sv.s, p.sv.s, min(TILE, p.S - tn), ldsV + (buf ^ 1) * TILE_BYTES);
+      stK.issue(tn, min(TILE, p.S - tn), ldsK + (buf ^ 1) * TILE_BYTES);
+      stV.issue(tn, min(TILE, p.S - tn), ldsV + (buf ^ 1) * TILE_BYTES);
     }
 
     const char* tk = ldsK + buf * TILE_BYTES;

@@ -272,7 +272,8 @@ def test_config3_keyformer_b1_h32_s4096_d128_tau1(gpu):
   ones = torch.ones(1, H, S, S, dtype=torch.float32, device=gpu)
   _, s_ones = ops.keyformer(qd, kd, vd, ones, tau=1.0)
   _, s_h2o = ops.h2o(qd, kd, vd)
-  assert torch.allclose(s_ones, s_h2o, rtol=1e-5, atol=1e-7)
+  # (the two paths differ in how the row sums are accumulated: fp32 exps vs the fp16 P fed to the MFMA)
+  assert torch.allclose(s_ones, s_h2o, rtol=2e-4, atol=1e-7)
   del ones
   # tensor noise, reference recipe and default tau, oracle on the first heads
   er = oracle.prepare_exp_rand(1, HS, S, S, seed=1)
