@@ -17,29 +17,34 @@
 #include "kernel_params.h"
 #include "noise.h"
 
+#include <type_traits>
+
 namespace ft {
 
 constexpr int kColBK = 128;  // keys per workgroup
 constexpr int kColBQ = 64;   // query rows per tile
 constexpr int kColThreads = 256;
 
-template <int D>
-constexpr int colstats_lds_bytes() {
-  return 2 * kColBQ * 2 * D + 2 * kColBQ * 8;
+// waves per SIMD the register budget is sized for: the packed-fp16 sum / sum-of-squares variants fit three
+template <typename T, bool EMU, int MODE>
+constexpr int colstats_waves_per_simd() {
+  return (__is_same(typename T::elem, _Float16) && EMU && (MODE == kStatSum || MODE == kStatSumSq)) ? 3 : 2;
 }
 
 template <typename T, int D, bool CAUSAL, bool EMU, int MODE>
-__global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const ColstatsKernelParams p) {
+__global__ void __launch_bounds__(kColThreads, colstats_waves_per_simd<T, EMU, MODE>()) colstats_kernel(const ColstatsKernelParams p) {
   constexpr int BK = kColBK, BQ = kColBQ, NT = kColThreads;
   constexpr int KSTEPS = D / 16;
   typedef TileGeom<D> G;
   typedef typename T::vec8 vec8;
   constexpr int TILE_BYTES = BQ * G::RB;
   constexpr bool KFM = (MODE == kStatKfTensor || MODE == kStatKfSeeded);
-  extern __shared__ __align__(16) char smem[];
-  char* ldsQ = smem;
-  float* ldsLse = reinterpret_cast<float*>(smem + 2 * TILE_BYTES);             // [2][BQ]
-  uint32_t* ldsRow = reinterpret_cast<uint32_t*>(smem + 2 * TILE_BYTES) + 2 * BQ;  // [2][BQ] noise row terms
+  constexpr bool kPacked = __is_same(typename T::elem, _Float16) && EMU;  // packed-fp16 rounding chain
+  // one LDS object per buffer: reads of one do not wait for the direct-to-LDS loads in flight into the other
+  __shared__ __align__(16) char ldsQ0[TILE_BYTES];
+  __shared__ __align__(16) char ldsQ1[TILE_BYTES];
+  __shared__ __align__(16) float ldsLse[2 * BQ];     // row normalisers of the current / next tile
+  __shared__ __align__(16) uint32_t ldsRow[2 * BQ];  // noise row terms (seeded KeyFormer)
 
   const int BH = p.B * p.H;
   const int bh = blockIdx.x % BH;
@@ -51,6 +56,7 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
   const int kj = j0 + wave * 32 + n;
   const int kj_c = kj < p.Skv ? kj : p.Skv - 1;
   const float POS_INF = __builtin_inff();
+  const float NEG_INF = -__builtin_inff();
 
   const uint16_t* kptr = p.k + b * p.sk.b + (int64_t)kj_c * p.sk.s + h * p.sk.h;
   vec8 kf[KSTEPS];
@@ -64,6 +70,10 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
   int i_begin = 0;
   if (CAUSAL) i_begin = max(0, j0 - p.off) / BQ * BQ;
   const int ntiles = (p.Sq - i_begin + BQ - 1) / BQ;  // <= 0 when no row sees this block
+  // leading tiles in which some (row, key) pair of this wave is above the diagonal
+  const int wave_key0 = j0 + wave * 32;
+  int n_masked = 0;
+  if (CAUSAL) n_masked = max(0, min(ntiles, (wave_key0 + 31 - p.off - i_begin + BQ - 1) / BQ));
 
   NoiseKeys nk = {0, 0};
   uint32_t b_j = 0;
@@ -74,33 +84,56 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
   }
   if (MODE == kStatKfTensor) er_col = p.exp_rand + b * p.er_sb + h * p.er_sh + kj_c;
 
-  float sum = 0.f, sumsq = 0.f;
   TileStager<D, BQ, NT, kRowSwizzle> stQ;
   stQ.init(qbase, p.sq.s);
+  uint32_t qoff[KSTEPS];  // Q row n (and n + 32 via an immediate), chunk 2t + g
+#pragma unroll
+  for (int t = 0; t < KSTEPS; ++t) qoff[t] = n * G::RB + (((2 * t + g) ^ G::row_swz(n)) << 4);
 
-  if (ntiles > 0) {
-    stQ.issue(i_begin, min(BQ, p.Sq - i_begin), ldsQ);
-    if (threadIdx.x < BQ) {
-      const int i = i_begin + threadIdx.x;
-      ldsLse[threadIdx.x] = i < p.Sq ? lse_bh[i] : POS_INF;
-      if (MODE == kStatKfSeeded) ldsRow[threadIdx.x] = noise_row(nk, (uint32_t)i);
+  float sum[4] = {0.f, 0.f, 0.f, 0.f}, sumsq[4] = {0.f, 0.f, 0.f, 0.f};  // independent chains
+
+  auto stage_q = [&](int t, char* dst) {
+    if (t < ntiles) stQ.issue(i_begin + t * BQ, min(BQ, p.Sq - (i_begin + t * BQ)), dst);
+  };
+  // rows of tile t: negated normaliser (-inf past Sq, so that those rows contribute exp2(-inf) = 0) and noise row term
+  auto stage_rows = [&](int t) {
+    if (t < ntiles && threadIdx.x < BQ) {
+      const int i = i_begin + t * BQ + threadIdx.x;
+      ldsLse[(t & 1) * BQ + threadIdx.x] = i < p.Sq ? -lse_bh[i] : NEG_INF;  // negated: one fma per logit
+      if (MODE == kStatKfSeeded) ldsRow[(t & 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)i);
     }
-  }
+  };
 
-  for (int it = 0; it < ntiles; ++it) {
-    const int i0 = i_begin + it * BQ;
-    const int buf = it & 1;
-    wait_vmem();
-    __syncthreads();
-
-    // rows of the next tile: normaliser (and noise row term) fetched now, parked in LDS at the end
-    float lse_next = POS_INF;
-    const bool has_next = it + 1 < ntiles;
-    if (has_next) {
-      const int in = i0 + BQ;
-      if (threadIdx.x < BQ && in + (int)threadIdx.x < p.Sq) lse_next = lse_bh[in + threadIdx.x];
+  // ---- S = Q K^T : [64 queries] x [32 keys] as two 32x32 blocks (16 LDS reads, 16 MFMAs)
+  auto qk = [&](float16v (&s)[2], const char* tq) {
+#pragma unroll
+    for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[mbk][r] = 0.f;
+    // operand ring: reads run kAhead k-steps ahead of the MFMAs that consume them
+    constexpr int kAhead = 3;
+    vec8 qa[kAhead + 1][2];
+#pragma unroll
+    for (int t = 0; t < kAhead; ++t)
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) qa[t][mbk] = *reinterpret_cast<const vec8*>(tq + qoff[t] + mbk * 32 * G::RB);
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t) {
+      if (t + kAhead < KSTEPS) {
+#pragma unroll
+        for (int mbk = 0; mbk < 2; ++mbk)
+          qa[(t + kAhead) % (kAhead + 1)][mbk] = *reinterpret_cast<const vec8*>(tq + qoff[t + kAhead] + mbk * 32 * G::RB);
+      }
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) s[mbk] = T::mfma(qa[t % (kAhead + 1)][mbk], kf[t], s[mbk]);
     }
+  };
 
+  // ---- probabilities of one tile from its raw scores, summed down the query axis in-lane
+  auto reduce_tile = [&](auto masked_tag, const float16v (&s)[2], int t) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const int buf = t & 1;
+    const int i0 = i_begin + t * BQ;
     float er[2][16];
     if (MODE == kStatKfTensor) {
 #pragma unroll
@@ -111,81 +144,134 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
           er[mbk][r] = (i < p.Sq) ? er_col[(int64_t)i * p.er_sr] : 1.f;
         }
     }
-
-    if (has_next) {
-      const int in = i0 + BQ;
-      stQ.issue(in, min(BQ, p.Sq - in), ldsQ + (buf ^ 1) * TILE_BYTES);
-    }
-
-    const int wave_key0 = j0 + wave * 32;
-    // every row of this tile is above the diagonal for all 32 keys of the wave
-    const bool skip = CAUSAL && (wave_key0 > i0 + BQ - 1 + p.off);
-    if (!skip) {
-      const char* tq = ldsQ + buf * TILE_BYTES;
-      float16v s_acc[2];
+    // key kj is hidden from row i0 + il when kj > i0 + il + off, i.e. il < lim
+    const int lim = kj - i0 - p.off - 4 * g;
 #pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
+    for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s_acc[mbk][r] = 0.f;
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int il0 = 32 * mbk + 8 * q4;  // + 4 g + e
+        const float4v nlse4 = *reinterpret_cast<const float4v*>(ldsLse + buf * BQ + il0 + 4 * g);
+        uint4v row4 = {0, 0, 0, 0};
+        if (MODE == kStatKfSeeded) row4 = *reinterpret_cast<const uint4v*>(ldsRow + buf * BQ + il0 + 4 * g);
+        float x[4];
+        if (kPacked && !KFM) {
 #pragma unroll
-      for (int t = 0; t < KSTEPS; ++t) {
-#pragma unroll
-        for (int mbk = 0; mbk < 2; ++mbk) {
-          vec8 qa = read_row_chunk<D, vec8>(tq, mbk * 32 + n, 2 * t + g);
-          s_acc[mbk] = T::mfma(qa, kf[t], s_acc[mbk]);
-        }
-      }
-
-      const bool need_mask = CAUSAL && (wave_key0 + 31 > i0 + p.off);
-#pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int il0 = 32 * mbk + 8 * q4 + 4 * g;
-          const float4v lse4 = *reinterpret_cast<const float4v*>(ldsLse + buf * BQ + il0);
-          uint4v row4 = {0, 0, 0, 0};
-          if (MODE == kStatKfSeeded) row4 = *reinterpret_cast<const uint4v*>(ldsRow + buf * BQ + il0);
+          for (int e = 0; e < 4; e += 2) {
+            const float2v a2 = {s[mbk][4 * q4 + e], s[mbk][4 * q4 + e + 1]};
+            const half2v h2 = __builtin_convertvector(a2, half2v);         // QK^T is an fp16 tensor in the reference
+            const _Float16 t0 = (_Float16)((float)h2[0] * p.logit_mul);    // ... divided by sqrt(D) in fp16
+            const _Float16 t1 = (_Float16)((float)h2[1] * p.logit_mul);
+            x[e] = __builtin_fmaf((float)t0, kLog2e, nlse4[e]);
+            x[e + 1] = __builtin_fmaf((float)t1, kLog2e, nlse4[e + 1]);
+          }
+        } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int r = 4 * q4 + e;
-            float x = s_acc[mbk][r];
+            float v = s[mbk][4 * q4 + e];
             if (EMU) {
-              x = T::to_float(T::from_float(x));
-              x = T::to_float(T::from_float(x * p.logit_mul));
-              x *= kLog2e;
+              v = T::to_float(T::from_float(v));
+              v = T::to_float(T::from_float(v * p.logit_mul));
+              v *= kLog2e;
             } else {
-              x *= p.logit_mul;
+              v *= p.logit_mul;
             }
             if (KFM) {
               float log2E;
               if (MODE == kStatKfTensor) {
-                log2E = __builtin_amdgcn_logf(er[mbk][r]);
+                log2E = __builtin_amdgcn_logf(er[mbk][4 * q4 + e]);
               } else {
                 const float u = noise_uniform(row4[e], b_j);
                 log2E = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(u));
               }
-              x = (x - log2E) * p.inv_tau;
+              v = (v - log2E) * p.inv_tau;
             }
-            float pr = __builtin_amdgcn_exp2f(x - lse4[e]);  // rows past Sq carry lse = +inf -> 0
-            if (need_mask && kj > i0 + il0 + e + p.off) pr = 0.f;
-            sum += pr;
-            if (MODE == kStatSumSq) sumsq = __builtin_fmaf(pr, pr, sumsq);
+            x[e] = v + nlse4[e];  // rows past Sq carry -inf -> p = 0
           }
         }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float xv = x[e];
+          if (MASKED) xv = (il0 + e < lim) ? NEG_INF : xv;
+          const float pr = __builtin_amdgcn_exp2f(xv);
+          sum[e] += pr;
+          if (MODE == kStatSumSq) sumsq[e] = __builtin_fmaf(pr, pr, sumsq[e]);
+        }
+      }
+  };
+  // operand reads a few MFMAs ahead of their consumers, MFMAs spread over the VALU work
+  auto sched_tile = [&]() {
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int i = 0; i < 2 * KSTEPS; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, KFM ? 24 : 12, 0);
     }
+  };
 
-    if (has_next && threadIdx.x < BQ) {
-      ldsLse[(buf ^ 1) * BQ + threadIdx.x] = lse_next;
-      if (MODE == kStatKfSeeded) ldsRow[(buf ^ 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)(i0 + BQ + threadIdx.x));
+  float16v S0[2], S1[2];
+  if (ntiles > 0) {
+    // ---- prologue: Q[0], Q[1] in flight; rows of tile 0; scores of tile 0
+    stage_q(0, ldsQ0);
+    stage_q(1, ldsQ1);
+    stage_rows(0);
+    wait_vmem();
+    __syncthreads();
+    qk(S0, ldsQ0);
+
+    // One iteration = one barrier.  On entry Q[t+1] has been requested and S0 (or S1) holds the scores of
+    // tile t; Q[t+2] is requested into the buffer whose tile was consumed one iteration ago.
+    int t = 0;
+    for (; t < n_masked; ++t) {
+      wait_vmem();
+      __syncthreads();
+      stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
+      stage_rows(t + 1);
+      // every row of this tile above the diagonal for all 32 keys of the wave: nothing to add
+      const bool skip = CAUSAL && (wave_key0 > i_begin + t * BQ + BQ - 1 + p.off);
+      if (!skip) reduce_tile(std::true_type{}, S0, t);
+      qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
+    }
+    // mask-free tiles, two per trip so that the score buffers swap roles without copies
+    if ((ntiles - t) & 1) {  // make the remainder even with one single step
+      wait_vmem();
+      __syncthreads();
+      stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
+      stage_rows(t + 1);
+      reduce_tile(std::false_type{}, S0, t);
+      qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
+      ++t;
+    }
+    const bool odd = t & 1;  // parity of the first tile of every pair
+    char* qa_buf = odd ? ldsQ1 : ldsQ0;  // holds tile t (consumed), refilled with t + 2
+    char* qb_buf = odd ? ldsQ0 : ldsQ1;  // holds tile t + 1
+    for (; t < ntiles; t += 2) {
+      wait_vmem();
+      __syncthreads();
+      stage_q(t + 2, qa_buf);
+      stage_rows(t + 1);
+      qk(S1, qb_buf);
+      reduce_tile(std::false_type{}, S0, t);
+      sched_tile();
+      wait_vmem();
+      __syncthreads();
+      stage_q(t + 3, qb_buf);
+      stage_rows(t + 2);
+      qk(S0, qa_buf);  // tile t + 2; past the last tile this reads stale LDS and is discarded
+      reduce_tile(std::false_type{}, S1, t + 1);
+      sched_tile();
     }
   }
 
-  sum += xchg32(sum);
-  if (MODE == kStatSumSq) sumsq += xchg32(sumsq);
+  float tot = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+  tot += xchg32(tot);
+  float totsq = (sumsq[0] + sumsq[1]) + (sumsq[2] + sumsq[3]);
+  if (MODE == kStatSumSq) totsq += xchg32(totsq);
   if (g == 0 && kj < p.Skv) {
     const int64_t idx = (int64_t)bh * p.Skv + kj;
-    p.colsum[idx] = sum;
-    if (MODE == kStatSumSq) p.colsumsq[idx] = sumsq;
+    p.colsum[idx] = tot;
+    if (MODE == kStatSumSq) p.colsumsq[idx] = totsq;
   }
 }
 
@@ -193,11 +279,9 @@ __global__ void __launch_bounds__(kColThreads, 2) colstats_kernel(const Colstats
 
 template <typename T, int D, bool CAUSAL, bool EMU, int MODE>
 static hipError_t launch_one(const ColstatsKernelParams& p, hipStream_t stream) {
-  auto kern = colstats_kernel<T, D, CAUSAL, EMU, MODE>;
-  constexpr int lds = colstats_lds_bytes<D>();
   const int nJB = (p.Skv + kColBK - 1) / kColBK;
   dim3 grid((unsigned)(nJB * p.B * p.H));
-  hipLaunchKernelGGL(kern, grid, dim3(kColThreads), lds, stream, p);
+  hipLaunchKernelGGL((colstats_kernel<T, D, CAUSAL, EMU, MODE>), grid, dim3(kColThreads), 0, stream, p);
   return hipGetLastError();
 }
 
