@@ -291,7 +291,8 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
     return fail(FT_EINVAL, "q, k, v, o must be 16-byte aligned");
   if (!stride_ok(a->sq) || !stride_ok(a->sk) || !stride_ok(a->sv) || !stride_ok(a->so))
     return fail(FT_EINVAL, "strides must be positive multiples of 8 elements with a contiguous head_dim axis");
-  if ((int64_t)a->Sq * a->sk.s * 2 >= 0x7fffffffLL || (int64_t)a->Sq * a->sv.s * 2 >= 0x7fffffffLL)
+  if ((int64_t)a->Sq * a->sq.s * 2 >= 0x7fffffffLL || (int64_t)a->Sq * a->sk.s * 2 >= 0x7fffffffLL ||
+      (int64_t)a->Sq * a->sv.s * 2 >= 0x7fffffffLL)
     return fail(FT_EUNSUPPORTED, "sequence stride too large: S * stride_s must stay below 2^30 elements");
   const size_t need = ft::linattn_workspace_bytes(*a, kind);
   if (!workspace || workspace_bytes < need)

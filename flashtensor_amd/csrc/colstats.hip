@@ -32,7 +32,7 @@ constexpr int colstats_waves_per_simd() {
 }
 
 template <typename T, int D, bool CAUSAL, bool EMU, int MODE>
-__global__ void __launch_bounds__(kColThreads, colstats_waves_per_simd<T, EMU, MODE>()) colstats_kernel(const ColstatsKernelParams p) {
+__global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, MODE>())) colstats_kernel(const ColstatsKernelParams p) {
   constexpr int BK = kColBK, BQ = kColBQ, NT = kColThreads;
   constexpr int KSTEPS = D / 16;
   typedef TileGeom<D> G;

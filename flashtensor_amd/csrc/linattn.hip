@@ -8,26 +8,39 @@
 // for the output product; EA reads it once) and writes O once.
 //
 // Three launches:
-//   1. kv_partial: a workgroup streams a chunk of tokens of one (b, h) in 128-token tiles through
-//      double-buffered LDS and accumulates the 64x64 matrix sum_s f(K[s,d]) V[s,e] with MFMA (both operands
+//   1. kv_partial: a workgroup owns a chunk of tokens of one (b, h); each of its four waves streams its
+//      own 16-token strips of K and V (and Q for SimA's norm) independently of the others: global loads
+//      into a rotating set of registers keep several strips in flight, a landed strip is written to a
+//      wave-private LDS buffer and read back transposed, so the loop has no workgroup barrier.  Per strip
+//      a wave accumulates the whole 64x64 matrix sum_s f(K[s,d]) V[s,e] with four MFMAs (both operands
 //      have the contraction axis = tokens strided in memory, so both come from ds_read_b64_tr_b16), plus
-//      the per-channel normalisers: EA an online (max, sum of exp) pair, SimA sum|K| and sum|Q|.
+//      the per-channel normalisers: EA an online (max, sum of exp) pair, SimA sum|K| and sum|Q|.  The
+//      four waves are combined through LDS at the end and one partial per chunk is written.
 //   2. merge: combines the chunks of one (b, h), folds every normaliser into the 64x64 matrix (the deferred
 //      division the reference's EquivalentTransform pass performs, EquivalentTransform.cpp:303-341) and
-//      stores it transposed as an fp16 hi/lo pair with a power-of-two scale, so that SimA's tiny values
-//      (~1e-6) neither underflow nor lose precision in fp16.
-//   3. out: O^T = W^T f(Q)^T per 32-token wave tile, with EA's per-token softmax over the 64 channels done
-//      in registers (a lane owns half a token row; one exchange with lane l ^ 32).
+//      stores it transposed as an fp16 hi/lo pair with a power-of-two scale per block of 16 output
+//      channels, so that SimA's tiny values (~1e-6) neither underflow nor lose precision in fp16.
+//   3. out: O^T = W^T f(Q)^T per 32-token wave tile.  A wave keeps W in registers for its whole chunk,
+//      streams Q strips the same way, does EA's per-token softmax over the 64 channels in registers (a
+//      lane owns half a token row; one exchange with lane l ^ 32) and turns the accumulator (lane =
+//      token) into full 128-byte output rows through a small LDS transpose.
+//
+// Direct-to-LDS loads are not used here on purpose: the compiler orders every LDS read after all
+// direct-to-LDS loads in flight unless it can prove they touch another LDS object, which drains a
+// multi-strip prefetch at each step; plain loads into registers are tracked exactly.
 #include "device_common.hpp"
 #include "kernel_params.h"
+#include <type_traits>
 #include "../../include/ft_abi.h"
 
 namespace ft {
 
 constexpr int kLinD = 64;
-constexpr int kLinTile = 128;     // tokens per staged tile
+constexpr int kLinTile = 128;     // chunk granularity in tokens
 constexpr int kLinThreads = 256;
+constexpr int kLinWaves = kLinThreads / 64;
 constexpr int kPartStride = kLinD * kLinD + 2 * kLinD;  // floats per (bh, chunk) partial
+constexpr int kNoSwizzle = 2;
 
 struct LinParams {
   const uint16_t* q;
@@ -37,12 +50,10 @@ struct LinParams {
   Strides3 sq, sk, sv, so;
   float* part;      // [BH][nch][kPartStride]
   uint16_t* w;      // [BH][2][64 e][64 d] fp16: hi, lo * 2^11
-  float* winv;      // [BH] 1 / scale
+  float* winv;      // [BH][4] 1 / scale of each block of 16 output channels
   int B, H, S;
   int nch;              // chunks per (b, h)
   int tiles_per_chunk;  // 128-token tiles per chunk
-  int normalize_q;
-  int out_f32;
 };
 
 static void lin_plan(const FtAttnArgs& a, int* nch, int* tpc) {
@@ -63,20 +74,72 @@ size_t linattn_workspace_bytes(const FtAttnArgs& a, int) {
   const size_t bh = (size_t)a.B * a.H;
   size_t bytes = bh * nch * kPartStride * sizeof(float);
   bytes += bh * 2 * kLinD * kLinD * sizeof(uint16_t);
-  bytes += bh * sizeof(float);
+  bytes += bh * 4 * sizeof(float);
   return (bytes + 255) & ~(size_t)255;
 }
 
+// Orders one wave's LDS traffic for the compiler; the hardware already executes a wave's LDS
+// instructions in order.
+__device__ __forceinline__ void wave_lds_order() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// One wave's private strip of ROWS tokens x 64 channels (128-byte rows): lane l moves the 16-byte chunk
+// l % 8 of rows l / 8 + 8 i, global -> registers -> LDS, so every load instruction covers 8 whole rows.
+// Rows past the end of the sequence re-read the last token (callers mask them).
+template <int ROWS, int SWZ>
+struct StripMover {
+  typedef TileGeom<kLinD> G;
+  static constexpr int ROUNDS = ROWS / 8;
+  const char* base;
+  int64_t row_bytes;
+  int last_row;
+  int r_lane;
+  int c16;
+  int lds_off[ROUNDS];
+
+  __device__ __forceinline__ void init(const uint16_t* base_, int64_t row_stride, int rows_total) {
+    base = reinterpret_cast<const char*>(base_);
+    row_bytes = row_stride * 2;
+    last_row = rows_total - 1;
+    const int lane = lane_id();
+    r_lane = lane >> 3;
+    c16 = (lane & 7) * 16;
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) {
+      const int r = it * 8 + r_lane;
+      const int cs = lane & 7;
+      const int c = SWZ == kRowSwizzle ? (cs ^ G::row_swz(r)) : SWZ == kTrSwizzle ? (cs ^ G::tr_swz(r)) : cs;
+      lds_off[it] = r * G::RB + c * 16;
+    }
+  }
+  __device__ __forceinline__ void load(int row0, uint4v (&regs)[ROUNDS]) const {
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) {
+      const int r = min(row0 + it * 8 + r_lane, last_row);
+      regs[it] = *reinterpret_cast<const uint4v*>(base + r * row_bytes + c16);
+    }
+  }
+  __device__ __forceinline__ void to_lds(const uint4v (&regs)[ROUNDS], char* lds_strip) const {
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) *reinterpret_cast<uint4v*>(lds_strip + lds_off[it]) = regs[it];
+  }
+};
+
 // ---------------------------------------------------------------------------------------------------
-template <bool EA>
+// NQ: also accumulate sum_s |Q| (SimA with normalised queries).
+template <bool EA, bool NQ>
 __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinParams p) {
-  constexpr int D = kLinD, NT = kLinThreads, TILE = kLinTile;
-  typedef TileGeom<D> G;
-  constexpr int TILE_BYTES = TILE * G::RB;  // 16 KB
-  extern __shared__ __align__(16) char smem[];
-  char* ldsK = smem;
-  char* ldsV = smem + 2 * TILE_BYTES;
-  float* ldsScratch = reinterpret_cast<float*>(smem + 4 * TILE_BYTES);  // [4 waves][32]
+  constexpr int D = kLinD, STEP = 16;
+  constexpr int P = 3;                        // strips in flight per wave
+  constexpr int STRIP = STEP * 2 * D;         // 2 KB
+  constexpr int R = STEP / 8;                 // 16-byte loads per lane, strip and tensor
+  __shared__ __align__(16) char s_kv[kLinWaves][2 * STRIP];  // wave-private K and V strips
+  __shared__ __align__(16) float s_x[2][D * D];              // end-of-kernel combine buffers
+  __shared__ float s_m[kLinWaves * D];
+  __shared__ float s_l[kLinWaves * D];
+  __shared__ float s_f[kLinWaves * D];
 
   const int BH = p.B * p.H;
   const int bh = blockIdx.x % BH;
@@ -84,212 +147,375 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
   const int b = bh / p.H, h = bh % p.H;
   const int lane = lane_id(), wave = wave_id();
   const int g = lane >> 5, n = lane & 31;
-  const int dblock = wave >> 1, eblock = wave & 1;
   const float NEG_INF = -__builtin_inff();
+  float* fac = s_f + wave * D;
+  char* tk = s_kv[wave];
+  char* tv = tk + STRIP;
 
-  const uint16_t* kbase = p.k + b * p.sk.b + h * p.sk.h;
-  const uint16_t* vbase = p.v + b * p.sv.b + h * p.sv.h;
-  const uint16_t* qbase = p.q + b * p.sq.b + h * p.sq.h;
+  const int tok_begin = ch * p.tiles_per_chunk * kLinTile;
+  const int tok_end = min(p.S, tok_begin + p.tiles_per_chunk * kLinTile);
+  const int nsteps = (tok_end - tok_begin + STEP - 1) / STEP;
+  const int nmine = nsteps > wave ? (nsteps - wave + kLinWaves - 1) / kLinWaves : 0;  // steps wave, wave + 4, ...
 
-  const int tok_begin = ch * p.tiles_per_chunk * TILE;
-  const int tok_end = min(p.S, tok_begin + p.tiles_per_chunk * TILE);
-  const int ntiles = (tok_end - tok_begin + TILE - 1) / TILE;
-
-  float16v acc;
+  float16v acc[2][2];  // [channel block of K][channel block of V]
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-  float m_run = NEG_INF;  // EA: running max of K[:, d] for this lane's channel d = 32 dblock + n
-  float l_run = 0.f;      // EA: sum of exp; SimA: sum |K|   (partial: this lane's token slots only)
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i >> 1][i & 1][r] = 0.f;
+  float m_run[2] = {NEG_INF, NEG_INF};  // EA: running max of K[:, d], d = 32 db + n
+  float l_run[2] = {0.f, 0.f};          // EA: sum of exp; SimA: sum |K|   (this lane's token slots only)
   float qabs[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) qabs[e] = 0.f;
 
-  TileStager<D, TILE, NT, kTrSwizzle> stK, stV;
-  stK.init(kbase, p.sk.s);
-  stV.init(vbase, p.sv.s);
-  stK.issue(tok_begin, min(TILE, p.S - tok_begin), ldsK);
-  stV.issue(tok_begin, min(TILE, p.S - tok_begin), ldsV);
+  StripMover<STEP, kTrSwizzle> mvK, mvV;
+  StripMover<STEP, kNoSwizzle> mvQ;
+  mvK.init(p.k + b * p.sk.b + h * p.sk.h, p.sk.s, p.S);
+  mvV.init(p.v + b * p.sv.b + h * p.sv.h, p.sv.s, p.S);
+  if (NQ) mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
 
-  for (int it = 0; it < ntiles; ++it) {
-    const int t0 = tok_begin + it * TILE;
-    const int buf = it & 1;
-    wait_vmem();
-    __syncthreads();
+  uint4v rk[P][R], rv[P][R], rq[P][R];  // strips in flight, indexed by compile-time slot
+  auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * STEP; };
+  auto fetch = [&](int i, auto slot_tag) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    const int row0 = strip_row0(i);
+    mvK.load(row0, rk[SLOT]);
+    mvV.load(row0, rv[SLOT]);
+    if (NQ) mvQ.load(row0, rq[SLOT]);
+  };
 
-    // SimA: |Q| partial sums straight from global memory (Q is not needed in LDS here)
-    if (!EA && p.normalize_q) {
-      const int c = threadIdx.x & 7;
+  // one strip, already in the wave's LDS buffer: TAIL = some of its tokens lie past the end
+  auto compute = [&](auto tail_tag, int t0) {
+    constexpr bool TAIL = decltype(tail_tag)::value;
+    half8 ka[2];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = t0 + (threadIdx.x >> 3) + 32 * i;
-        if (tok < p.S) {
-          half8 qv = *reinterpret_cast<const half8*>(qbase + (int64_t)tok * p.sq.s + c * 8);
+    for (int db = 0; db < 2; ++db) ka[db] = read_tr_operand<D, half8>(tk, 0, 32 * db);
+    half8 vb[2];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) qabs[e] += __builtin_fabsf((float)qv[e]);
-        }
-      }
-    }
-
-    if (it + 1 < ntiles) {
-      const int tn = t0 + TILE;
-      stK.issue(tn, min(TILE, p.S - tn), ldsK + (buf ^ 1) * TILE_BYTES);
-      stV.issue(tn, min(TILE, p.S - tn), ldsV + (buf ^ 1) * TILE_BYTES);
-    }
-
-    const char* tk = ldsK + buf * TILE_BYTES;
-    const char* tv = ldsV + buf * TILE_BYTES;
-    const bool tail = t0 + TILE > p.S;
-
-    half8 ka[TILE / 16];
+    for (int eb = 0; eb < 2; ++eb) vb[eb] = read_tr_operand<D, half8>(tv, 0, 32 * eb);
+    bool dead[8];  // token slot s of this lane is past the end
 #pragma unroll
-    for (int ks = 0; ks < TILE / 16; ++ks) ka[ks] = read_tr_operand<D, half8>(tk, 16 * ks, 32 * dblock);
+    for (int s = 0; s < 8; ++s) dead[s] = TAIL && t0 + 4 * g + (s & 3) + ((s >> 2) << 3) >= p.S;
 
     if (EA) {
-      float tmax = NEG_INF;
+      float m_new[2];
 #pragma unroll
-      for (int ks = 0; ks < TILE / 16; ++ks)
+      for (int db = 0; db < 2; ++db) {
+        float mx;
+        if (TAIL) {
+          mx = NEG_INF;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const int tok = t0 + 16 * ks + 4 * g + (s & 3) + ((s >> 2) << 3);
-          const float x = (float)ka[ks][s];
-          tmax = fmaxf(tmax, (tail && tok >= p.S) ? NEG_INF : x);
+          for (int s = 0; s < 8; ++s) mx = fmaxf(mx, dead[s] ? NEG_INF : (float)ka[db][s]);
+        } else {
+          half2v hm = __builtin_elementwise_max(__builtin_shufflevector(ka[db], ka[db], 0, 1), __builtin_shufflevector(ka[db], ka[db], 2, 3));
+          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(ka[db], ka[db], 4, 5));
+          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(ka[db], ka[db], 6, 7));
+          mx = fmaxf((float)hm[0], (float)hm[1]);
         }
-      tmax = fmaxf(tmax, xchg32(tmax));
-      const float m_new = fmaxf(m_run, tmax);
-      if (__any(m_new > m_run)) {
-        const float f = __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
-        l_run *= f;
-        // move the per-channel factor from "lane = channel" to the accumulator's "register = channel"
-        float* sc = ldsScratch + wave * 32;
-        if (g == 0) sc[n] = f;
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const float4v f4 = *reinterpret_cast<const float4v*>(sc + 8 * q4 + 4 * g);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[4 * q4 + e] *= f4[e];
-        }
+        mx = fmaxf(mx, xchg32(mx));
+        m_new[db] = fmaxf(m_run[db], mx);
       }
-      m_run = m_new;
-      const float mb = m_new * kLog2e;
+      if (__any(m_new[0] > m_run[0] || m_new[1] > m_run[1])) {
+        // move the per-channel factor from "lane = channel" to the accumulator's "register = channel"
 #pragma unroll
-      for (int ks = 0; ks < TILE / 16; ++ks)
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const int tok = t0 + 16 * ks + 4 * g + (s & 3) + ((s >> 2) << 3);
-          float pe = __builtin_amdgcn_exp2f(__builtin_fmaf((float)ka[ks][s], kLog2e, -mb));
-          if (tail && tok >= p.S) pe = 0.f;
-          const _Float16 ph = (_Float16)pe;
-          ka[ks][s] = ph;
-          l_run += (float)ph;
+        for (int db = 0; db < 2; ++db) {
+          const float f = __builtin_amdgcn_exp2f((m_run[db] - m_new[db]) * kLog2e);
+          l_run[db] *= f;
+          if (g == 0) fac[32 * db + n] = f;
+          m_run[db] = m_new[db];
         }
+        wave_lds_order();
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const float4v f4 = *reinterpret_cast<const float4v*>(fac + 32 * db + 8 * q4 + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              acc[db][0][4 * q4 + e] *= f4[e];
+              acc[db][1][4 * q4 + e] *= f4[e];
+            }
+          }
+        wave_lds_order();
+      }
+      const half2v ones = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+      for (int db = 0; db < 2; ++db) {
+        const float mb = m_run[db] * kLog2e;
+        uint4v pw;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf((float)ka[db][2 * j], kLog2e, -mb));
+          float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf((float)ka[db][2 * j + 1], kLog2e, -mb));
+          if (dead[2 * j]) e0 = 0.f;
+          if (dead[2 * j + 1]) e1 = 0.f;
+          const float2v e2 = {e0, e1};
+          const half2v ph = __builtin_convertvector(e2, half2v);
+          l_run[db] = __builtin_amdgcn_fdot2(ph, ones, l_run[db], false);  // sum of the fp16 values the MFMA consumes
+          pw[j] = __builtin_bit_cast(uint32_t, ph);
+        }
+        ka[db] = __builtin_bit_cast(half8, pw);
+      }
     } else {
 #pragma unroll
-      for (int ks = 0; ks < TILE / 16; ++ks)
+      for (int db = 0; db < 2; ++db)
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-          const int tok = t0 + 16 * ks + 4 * g + (s & 3) + ((s >> 2) << 3);
-          if (tail && tok >= p.S) ka[ks][s] = (_Float16)0.f;
-          l_run += __builtin_fabsf((float)ka[ks][s]);
+          if (dead[s]) ka[db][s] = (_Float16)0.f;
+          l_run[db] += __builtin_fabsf((float)ka[db][s]);
         }
     }
-
 #pragma unroll
-    for (int ks = 0; ks < TILE / 16; ++ks) {
-      half8 vb = read_tr_operand<D, half8>(tv, 16 * ks, 32 * eblock);
-      acc = F16::mfma(ka[ks], vb, acc);
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int eb = 0; eb < 2; ++eb) acc[db][eb] = F16::mfma(ka[db], vb[eb], acc[db][eb]);
+  };
+
+  // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P
+  // (always fetched: rows are clamped), then consume the parked strip
+  auto step = [&](int i, auto slot_tag) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    const int t0 = strip_row0(i);
+    const bool tail = t0 + STEP > p.S;
+    wave_lds_order();
+    mvK.to_lds(rk[SLOT], tk);
+    mvV.to_lds(rv[SLOT], tv);
+    if (NQ) {
+      // a lane holds channels 8 (lane % 8) + [0..7] of rows lane / 8 (+ 8) of the strip
+#pragma unroll
+      for (int it = 0; it < R; ++it) {
+        const half8 qv = __builtin_bit_cast(half8, rq[SLOT][it]);
+        const bool live = !tail || t0 + it * 8 + (lane >> 3) < p.S;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qabs[e] += live ? __builtin_fabsf((float)qv[e]) : 0.f;
+      }
+    }
+    fetch(i + P, slot_tag);
+    wave_lds_order();
+    if (tail)
+      compute(std::true_type{}, t0);
+    else
+      compute(std::false_type{}, t0);
+  };
+
+  fetch(0, std::integral_constant<int, 0>{});
+  fetch(1, std::integral_constant<int, 1>{});
+  fetch(2, std::integral_constant<int, 2>{});
+  static_assert(P == 3, "the strip loop is unrolled over three register slots");
+  for (int i = 0; i < nmine;) {
+    step(i, std::integral_constant<int, 0>{});
+    if (++i >= nmine) break;
+    step(i, std::integral_constant<int, 1>{});
+    if (++i >= nmine) break;
+    step(i, std::integral_constant<int, 2>{});
+    ++i;
+  }
+
+  // ---- combine the four waves
+#pragma unroll
+  for (int db = 0; db < 2; ++db) {
+    l_run[db] += xchg32(l_run[db]);
+    if (g == 0) {
+      s_m[wave * D + 32 * db + n] = m_run[db];
+      s_l[wave * D + 32 * db + n] = l_run[db];
     }
   }
+  if (NQ) {
+    // |Q| column sums: a lane holds channels 8 (lane % 8) + [0..7] of its row group; fold the 8 row groups
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float s = qabs[e];
+      s += __shfl_xor(s, 8);
+      s += __shfl_xor(s, 16);
+      s += __shfl_xor(s, 32);
+      qabs[e] = s;
+    }
+    if (lane < 8) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) fac[lane * 8 + e] = qabs[e];
+    }
+  }
+  __syncthreads();
+  if (EA) {
+    // bring every wave's matrix to the common per-channel maximum
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d0 = 32 * db + 8 * q4 + 4 * g;
+        float4v mall = *reinterpret_cast<const float4v*>(s_m + d0);
+#pragma unroll
+        for (int w = 1; w < kLinWaves; ++w) {
+          const float4v mw = *reinterpret_cast<const float4v*>(s_m + w * D + d0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) mall[e] = fmaxf(mall[e], mw[e]);
+        }
+        const float4v mine = *reinterpret_cast<const float4v*>(s_m + wave * D + d0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float f = __builtin_amdgcn_exp2f((mine[e] - mall[e]) * kLog2e);
+          acc[db][0][4 * q4 + e] *= f;
+          acc[db][1][4 * q4 + e] *= f;
+        }
+      }
+  }
+  // pairwise tree: waves 2, 3 -> waves 0, 1, then wave 1 -> wave 0
+  float* xa = s_x[0];
+  float* xb = s_x[1];
+  auto put = [&](float* dst) {
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int eb = 0; eb < 2; ++eb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst[((2 * db + eb) * 16 + r) * 64 + lane] = acc[db][eb][r];
+  };
+  auto add = [&](const float* src) {
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int eb = 0; eb < 2; ++eb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[db][eb][r] += src[((2 * db + eb) * 16 + r) * 64 + lane];
+  };
+  if (wave == 2) put(xa);
+  if (wave == 3) put(xb);
+  __syncthreads();
+  if (wave == 0) add(xa);
+  if (wave == 1) add(xb);
+  __syncthreads();
+  if (wave == 1) put(xa);
+  __syncthreads();
 
-  // ---- write the partial
   float* part = p.part + ((int64_t)bh * p.nch + ch) * kPartStride;
+  if (wave == 0) {
+    add(xa);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int d = 32 * dblock + 8 * (r >> 2) + 4 * g + (r & 3);
-    part[d * D + 32 * eblock + n] = acc[r];
-  }
-  l_run += xchg32(l_run);
-  if (eblock == 0 && g == 0) {
-    const int d = 32 * dblock + n;
-    part[D * D + d] = EA ? m_run : l_run;
-    if (EA) part[D * D + D + d] = l_run;
-  }
-  if (!EA) {
-    __syncthreads();  // tiles are dead: reuse LDS for the |Q| reduction
-    float* red = reinterpret_cast<float*>(smem);  // [32 row groups][64 channels]
-    const int c = threadIdx.x & 7, rg = threadIdx.x >> 3;
+    for (int db = 0; db < 2; ++db)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) red[rg * D + c * 8 + e] = qabs[e];
-    __syncthreads();
-    if (threadIdx.x < D) {
-      float s = 0.f;
-      for (int i = 0; i < 32; ++i) s += red[i * D + threadIdx.x];
-      part[D * D + D + threadIdx.x] = s;
+      for (int eb = 0; eb < 2; ++eb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = 32 * db + 8 * (r >> 2) + 4 * g + (r & 3);
+          part[d * D + 32 * eb + n] = acc[db][eb][r];
+        }
+  } else if (wave == 1) {
+    const int d = lane;
+    if (EA) {
+      float M = s_m[d];
+#pragma unroll
+      for (int w = 1; w < kLinWaves; ++w) M = fmaxf(M, s_m[w * D + d]);
+      float L = 0.f;
+#pragma unroll
+      for (int w = 0; w < kLinWaves; ++w) L += __builtin_amdgcn_exp2f((s_m[w * D + d] - M) * kLog2e) * s_l[w * D + d];
+      part[D * D + d] = M;
+      part[D * D + D + d] = L;
+    } else {
+      float nk = 0.f, nq = 0.f;
+#pragma unroll
+      for (int w = 0; w < kLinWaves; ++w) {
+        nk += s_l[w * D + d];
+        if (NQ) nq += s_f[w * D + d];
+      }
+      part[D * D + d] = nk;
+      part[D * D + D + d] = nq;
     }
   }
 }
 
 // ---------------------------------------------------------------------------------------------------
+// One workgroup per (b, h, block of 16 output channels).
 template <bool EA>
-__global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinParams p) {
-  constexpr int D = kLinD;
+__global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinParams p, int normalize_q) {
+  constexpr int D = kLinD, EB = 16, TS = D + 8;
   __shared__ float s_scale[D];   // per-channel factor applied to the summed matrix
+  __shared__ float s_big[D];     // EA: global max per channel
   __shared__ float s_w[16][D];   // EA: per-chunk weights exp(m_c - M), up to 16 chunks at a time
   __shared__ float s_red[kLinThreads];
-  const int bh = blockIdx.x;
+  __shared__ __align__(16) uint16_t s_t[2][EB][TS];  // hi / lo, transposed for 16-byte row stores
+  const int bh = blockIdx.x >> 2;
+  const int qr = blockIdx.x & 3;
   const float* part = p.part + (int64_t)bh * p.nch * kPartStride;
   const int t = threadIdx.x;
 
-  float accv[16];
+  float accv[4] = {0.f, 0.f, 0.f, 0.f};
+  int pidx[4], drow[4];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) accv[i] = 0.f;
-  float gmax = -__builtin_inff();
+  for (int i = 0; i < 4; ++i) {
+    const int idx = t + i * kLinThreads;  // d = idx / 16, e = 16 qr + idx % 16
+    drow[i] = idx / EB;
+    pidx[i] = drow[i] * D + EB * qr + idx % EB;
+  }
 
+  // per-channel statistics: four thread groups split the chunks, then fold through LDS
+  const int sd = t & (D - 1), cg = t >> 6;
+  const float* stat = part + D * D + sd;
   if (EA) {
+    float M = -__builtin_inff();
+    for (int c = cg; c < p.nch; c += 4) M = fmaxf(M, stat[c * kPartStride]);
+    s_red[t] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(s_red[sd], s_red[D + sd]), fmaxf(s_red[2 * D + sd], s_red[3 * D + sd]));
+    float L = 0.f;
+    for (int c = cg; c < p.nch; c += 4)
+      L += __builtin_amdgcn_exp2f((stat[c * kPartStride] - M) * kLog2e) * stat[c * kPartStride + D];
+    __syncthreads();
+    s_red[t] = L;
+    __syncthreads();
     if (t < D) {
-      float M = -__builtin_inff();
-      for (int c = 0; c < p.nch; ++c) M = fmaxf(M, part[c * kPartStride + D * D + t]);
-      float L = 0.f;
-      for (int c = 0; c < p.nch; ++c)
-        L += __builtin_amdgcn_exp2f((part[c * kPartStride + D * D + t] - M) * kLog2e) * part[c * kPartStride + D * D + D + t];
-      s_scale[t] = 1.f / L;
-      s_red[t] = M;
+      s_scale[t] = 1.f / (s_red[t] + s_red[D + t] + s_red[2 * D + t] + s_red[3 * D + t]);
+      s_big[t] = M;
     }
     __syncthreads();
-    for (int c0 = 0; c0 < p.nch; c0 += 16) {
-      const int cn = min(16, p.nch - c0);
+  } else {
+    float nk = 0.f, nq = 0.f;
+    for (int c = cg; c < p.nch; c += 4) {
+      nk += stat[c * kPartStride];
+      nq += stat[c * kPartStride + D];
+    }
+    s_red[t] = nk;
+    s_w[cg][sd] = nq;
+    __syncthreads();
+    if (t < D) {
+      nk = s_red[t] + s_red[D + t] + s_red[2 * D + t] + s_red[3 * D + t];
+      nq = s_w[0][t] + s_w[1][t] + s_w[2][t] + s_w[3][t];
+      s_scale[t] = 1.f / (normalize_q ? nk * nq : nk);
+    }
+    __syncthreads();
+  }
+  // weighted sum of the chunk matrices, four chunks (16 independent loads per thread) at a time
+  for (int c0 = 0; c0 < p.nch; c0 += 16) {
+    const int cn = min(16, p.nch - c0);
+    if (EA) {
       for (int i = t; i < cn * D; i += kLinThreads) {
         const int c = i / D, d = i % D;
-        s_w[c][d] = __builtin_amdgcn_exp2f((part[(c0 + c) * kPartStride + D * D + d] - s_red[d]) * kLog2e);
+        s_w[c][d] = __builtin_amdgcn_exp2f((part[(c0 + c) * kPartStride + D * D + d] - s_big[d]) * kLog2e);
       }
       __syncthreads();
-      for (int c = 0; c < cn; ++c)
+    }
+    for (int c = 0; c < cn; c += 4) {
+      float v[4][4];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int idx = t + i * kLinThreads;  // d = idx / 64, e = idx % 64
-          accv[i] += s_w[c][idx / D] * part[(c0 + c) * kPartStride + idx];
+      for (int u = 0; u < 4; ++u) {
+        const int cc = c0 + min(c + u, cn - 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[u][i] = part[cc * kPartStride + pidx[i]];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (c + u < cn) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) accv[i] += (EA ? s_w[c + u][drow[i]] : 1.f) * v[u][i];
         }
-      __syncthreads();
     }
-  } else {
-    if (t < D) {
-      float nk = 0.f, nq = 0.f;
-      for (int c = 0; c < p.nch; ++c) {
-        nk += part[c * kPartStride + D * D + t];
-        nq += part[c * kPartStride + D * D + D + t];
-      }
-      s_scale[t] = 1.f / (p.normalize_q ? nk * nq : nk);
-    }
-    __syncthreads();
-    for (int c = 0; c < p.nch; ++c)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) accv[i] += part[c * kPartStride + t + i * kLinThreads];
+    if (EA) __syncthreads();
   }
+  float gmax = 0.f;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    accv[i] *= s_scale[(t + i * kLinThreads) / D];
+  for (int i = 0; i < 4; ++i) {
+    accv[i] *= s_scale[drow[i]];
     gmax = fmaxf(gmax, __builtin_fabsf(accv[i]));
   }
-  __syncthreads();
   s_red[t] = gmax;
   __syncthreads();
   for (int s = kLinThreads / 2; s > 0; s >>= 1) {
@@ -297,37 +523,61 @@ __global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinPar
     __syncthreads();
   }
   gmax = s_red[0];
-  // power-of-two scale that puts the largest entry in [2^13, 2^14)
+  // power-of-two scale that puts the largest entry of the block in [2^13, 2^14)
   int ex = 0;
   if (gmax > 0.f && gmax < __builtin_inff()) ex = 13 - (int)__builtin_floorf(__builtin_log2f(gmax));
   ex = max(-100, min(100, ex));
   const float scale = __builtin_ldexpf(1.f, ex);
-  if (t == 0) p.winv[bh] = __builtin_ldexpf(1.f, -ex);
-  uint16_t* w = p.w + (int64_t)bh * 2 * D * D;
+  if (t == 0) p.winv[bh * 4 + qr] = __builtin_ldexpf(1.f, -ex);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const int idx = t + i * kLinThreads;
-    const int d = idx / D, e = idx % D;
     const float x = accv[i] * scale;
     const _Float16 hi = (_Float16)x;
     const _Float16 lo = (_Float16)((x - (float)hi) * 2048.f);
-    w[e * D + d] = __builtin_bit_cast(uint16_t, hi);
-    w[D * D + e * D + d] = __builtin_bit_cast(uint16_t, lo);
+    s_t[0][idx % EB][drow[i]] = __builtin_bit_cast(uint16_t, hi);
+    s_t[1][idx % EB][drow[i]] = __builtin_bit_cast(uint16_t, lo);
+  }
+  __syncthreads();
+  {
+    const int hl = t >> 7, e = (t & 127) >> 3, c = t & 7;
+    uint16_t* w = p.w + (int64_t)bh * 2 * D * D + hl * D * D + (EB * qr + e) * D + c * 8;
+    *reinterpret_cast<uint4v*>(w) = *reinterpret_cast<const uint4v*>(&s_t[hl][e][c * 8]);
   }
 }
 
 // ---------------------------------------------------------------------------------------------------
 template <bool EA, bool F32OUT>
 __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinParams p) {
-  constexpr int D = kLinD;
+  constexpr int D = kLinD, SUB = 32;
+  constexpr int P = 2;                           // Q strips in flight per wave
+  constexpr int STRIP = SUB * 2 * D;             // 4 KB
+  constexpr int R = SUB / 8;                     // 16-byte loads per lane and strip
+  constexpr int OROW = F32OUT ? 272 : 144;       // padded output row in the transpose buffer (bytes)
+  constexpr int SL = SUB * D * (F32OUT ? 4 : 2) / 1024;  // 16-byte row stores per strip and lane
+  __shared__ __align__(16) char s_q[kLinWaves][STRIP];       // wave-private Q strip
+  __shared__ __align__(16) char otr[kLinWaves * SUB * OROW]; // wave-private output transpose buffers
+
   const int BH = p.B * p.H;
   const int bh = blockIdx.x % BH;
-  const int tb = blockIdx.x / BH;
+  const int ch = blockIdx.x / BH;
   const int b = bh / p.H, h = bh % p.H;
   const int lane = lane_id(), wave = wave_id();
   const int g = lane >> 5, n = lane & 31;
-  const int tok = tb * 128 + wave * 32 + n;
-  const int tok_c = tok < p.S ? tok : p.S - 1;
+  char* ost = otr + wave * SUB * OROW;
+  char* tq = s_q[wave];
+
+  const int tok_begin = ch * p.tiles_per_chunk * kLinTile;
+  const int tok_end = min(p.S, tok_begin + p.tiles_per_chunk * kLinTile);
+  const int nsub = (tok_end - tok_begin + SUB - 1) / SUB;
+  const int nmine = nsub > wave ? (nsub - wave + kLinWaves - 1) / kLinWaves : 0;
+
+  StripMover<SUB, kRowSwizzle> mvQ;
+  mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
+  uint4v rq[P][R];  // strips in flight, indexed by compile-time slot
+  auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * SUB; };
+  mvQ.load(strip_row0(0), rq[0]);
+  mvQ.load(strip_row0(1), rq[1]);
 
   // A operand: W^T[e][d], hi and lo, rows e = 32 eb + n, contraction slots d = 16 t + 8 g + [0..7]
   const uint16_t* w = p.w + (int64_t)bh * 2 * D * D;
@@ -337,61 +587,85 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       whi[eb][t] = *reinterpret_cast<const half8*>(w + (32 * eb + n) * D + 16 * t + 8 * g);
-      wlo[eb][t] = *reinterpret_cast<const half8*>(w + D * D + (32 * eb + n) * D + 16 * t + 8 * g);
+      if (F32OUT) wlo[eb][t] = *reinterpret_cast<const half8*>(w + D * D + (32 * eb + n) * D + 16 * t + 8 * g);
     }
-  const float winv = p.winv[bh];
+  float winv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) winv[i] = p.winv[bh * 4 + i];
 
-  // B operand: f(Q)^T, column = token n, same contraction slots
-  const uint16_t* qrow = p.q + b * p.sq.b + (int64_t)tok_c * p.sq.s + h * p.sq.h;
-  half8 qf[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) qf[t] = *reinterpret_cast<const half8*>(qrow + 16 * t + 8 * g);
+  char* obase = static_cast<char*>(p.o) + (b * p.so.b + h * p.so.h) * (int64_t)(F32OUT ? 4 : 2);
+  const int64_t orow_bytes = p.so.s * (int64_t)(F32OUT ? 4 : 2);
 
-  if (EA) {
-    float x[4][8];
-    float mx = -__builtin_inff();
+  // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P
+  // (always fetched: rows are clamped), then consume the parked strip
+  auto step = [&](int i, auto slot_tag) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    const int t0 = strip_row0(i);
+    wave_lds_order();
+    mvQ.to_lds(rq[SLOT], tq);
+    mvQ.load(strip_row0(i + P), rq[SLOT]);
+    wave_lds_order();
+
+    // B operand: f(Q)^T, column = token n, same contraction slots
+    half8 qf[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 4; ++t) qf[t] = read_row_chunk<D, half8>(tq, n, 2 * t + g);
+
+    // EA: softmax over the 64 channels of the token.  The operand is the fp16 value of exp(q - max); the
+    // division by the row sum (taken over those rounded values) is applied to the fp32 result.
+    float inv = 1.f;
+    if (EA) {
+      half2v hm = __builtin_shufflevector(qf[0], qf[0], 0, 1);
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        x[t][s] = (float)qf[t][s] * kLog2e;
-        mx = fmaxf(mx, x[t][s]);
+      for (int t = 0; t < 4; ++t) {
+        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 0, 1));
+        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 2, 3));
+        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 4, 5));
+        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 6, 7));
       }
-    mx = fmaxf(mx, xchg32(mx));
-    float sum = 0.f;
+      float mx = fmaxf((float)hm[0], (float)hm[1]);
+      mx = fmaxf(mx, xchg32(mx));
+      const float mb = mx * kLog2e;
+      const half2v ones = {(_Float16)1.f, (_Float16)1.f};
+      float sum = 0.f;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 4; ++t) {
+        uint4v pw;
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        x[t][s] = __builtin_amdgcn_exp2f(x[t][s] - mx);
-        sum += x[t][s];
+        for (int j = 0; j < 4; ++j) {
+          const float2v e2 = {__builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j], kLog2e, -mb)),
+                              __builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j + 1], kLog2e, -mb))};
+          const half2v ph = __builtin_convertvector(e2, half2v);
+          sum = __builtin_amdgcn_fdot2(ph, ones, sum, false);
+          pw[j] = __builtin_bit_cast(uint32_t, ph);
+        }
+        qf[t] = __builtin_bit_cast(half8, pw);
       }
-    sum += xchg32(sum);
-    const float inv = 1.f / sum;
+      sum += xchg32(sum);
+      inv = 1.f / sum;
+    }
+
+    // W as hi + lo / 2^11 only where the output can show the difference (fp32)
+    float16v ahi[2], alo[2];
+#pragma unroll
+    for (int eb = 0; eb < 2; ++eb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        ahi[eb][r] = 0.f;
+        alo[eb][r] = 0.f;
+      }
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int s = 0; s < 8; ++s) qf[t][s] = (_Float16)(x[t][s] * inv);
-  }
+      for (int eb = 0; eb < 2; ++eb) {
+        ahi[eb] = F16::mfma(whi[eb][t], qf[t], ahi[eb]);
+        if (F32OUT) alo[eb] = F16::mfma(wlo[eb][t], qf[t], alo[eb]);
+      }
+    float osc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) osc[i] = winv[i] * inv;
 
-  float16v ahi[2], alo[2];
-#pragma unroll
-  for (int eb = 0; eb < 2; ++eb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      ahi[eb][r] = 0.f;
-      alo[eb][r] = 0.f;
-    }
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int eb = 0; eb < 2; ++eb) {
-      ahi[eb] = F16::mfma(whi[eb][t], qf[t], ahi[eb]);
-      alo[eb] = F16::mfma(wlo[eb][t], qf[t], alo[eb]);
-    }
-
-  if (tok < p.S) {
-    const int64_t off = b * p.so.b + (int64_t)tok * p.so.s + h * p.so.h;
+    // accumulator (lane = token, registers = channels) -> padded [token][channel] rows in LDS
 #pragma unroll
     for (int eb = 0; eb < 2; ++eb)
 #pragma unroll
@@ -399,17 +673,37 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
         const int e0 = 32 * eb + 8 * q4 + 4 * g;
         float y[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) y[e] = (ahi[eb][4 * q4 + e] + alo[eb][4 * q4 + e] * (1.f / 2048.f)) * winv;
+        for (int e = 0; e < 4; ++e)
+          y[e] = (F32OUT ? ahi[eb][4 * q4 + e] + alo[eb][4 * q4 + e] * (1.f / 2048.f) : ahi[eb][4 * q4 + e]) * osc[2 * eb + (q4 >> 1)];
         if (F32OUT) {
           float4v o4 = {y[0], y[1], y[2], y[3]};
-          *reinterpret_cast<float4v*>(static_cast<float*>(p.o) + off + e0) = o4;
+          *reinterpret_cast<float4v*>(ost + n * OROW + e0 * 4) = o4;
         } else {
           uint2 pk;
           pk.x = (uint32_t)F16::from_float(y[0]) | ((uint32_t)F16::from_float(y[1]) << 16);
           pk.y = (uint32_t)F16::from_float(y[2]) | ((uint32_t)F16::from_float(y[3]) << 16);
-          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.o) + off + e0) = pk;
+          *reinterpret_cast<uint2*>(ost + n * OROW + e0 * 2) = pk;
         }
       }
+    wave_lds_order();
+    // whole rows back out: 16 bytes per lane, 8 (fp16) or 16 (fp32) lanes per token
+    constexpr int LPR = F32OUT ? 16 : 8;
+#pragma unroll
+    for (int j = 0; j < SL; ++j) {
+      const int r = j * (64 / LPR) + lane / LPR;
+      const int c = lane % LPR;
+      const uint4v val = *reinterpret_cast<const uint4v*>(ost + r * OROW + c * 16);
+      if (t0 + r < p.S) *reinterpret_cast<uint4v*>(obase + (int64_t)(t0 + r) * orow_bytes + c * 16) = val;
+    }
+    wave_lds_order();
+  };
+
+  static_assert(P == 2, "the strip loop is unrolled over two register slots");
+  for (int i = 0; i < nmine;) {
+    step(i, std::integral_constant<int, 0>{});
+    if (++i >= nmine) break;
+    step(i, std::integral_constant<int, 1>{});
+    ++i;
   }
 }
 
@@ -429,8 +723,8 @@ hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int ou
   p.S = a.Sq;
   lin_plan(a, &p.nch, &p.tiles_per_chunk);
   const bool ea = kind == FT_OP_EA;
-  p.normalize_q = ea ? 0 : normalize_q;
-  p.out_f32 = out_dtype == FT_F32;
+  const bool nq = !ea && normalize_q;
+  const bool f32 = out_dtype == FT_F32;
   const size_t bh = (size_t)a.B * a.H;
   char* base = static_cast<char*>(ws);
   p.part = reinterpret_cast<float*>(base);
@@ -439,39 +733,32 @@ hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int ou
   base += bh * 2 * kLinD * kLinD * sizeof(uint16_t);
   p.winv = reinterpret_cast<float*>(base);
 
-  constexpr int lds1 = 4 * kLinTile * 2 * kLinD + 4 * 32 * 4;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linattn_kv_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(linattn_kv_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
   const dim3 grid1((unsigned)(bh * p.nch)), blk(kLinThreads);
   if (ea)
-    hipLaunchKernelGGL(linattn_kv_kernel<true>, grid1, blk, lds1, s, p);
+    hipLaunchKernelGGL((linattn_kv_kernel<true, false>), grid1, blk, 0, s, p);
+  else if (nq)
+    hipLaunchKernelGGL((linattn_kv_kernel<false, true>), grid1, blk, 0, s, p);
   else
-    hipLaunchKernelGGL(linattn_kv_kernel<false>, grid1, blk, lds1, s, p);
+    hipLaunchKernelGGL((linattn_kv_kernel<false, false>), grid1, blk, 0, s, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
+  const dim3 grid2((unsigned)(bh * 4));
   if (ea)
-    hipLaunchKernelGGL(linattn_merge_kernel<true>, dim3((unsigned)bh), blk, 0, s, p);
+    hipLaunchKernelGGL(linattn_merge_kernel<true>, grid2, blk, 0, s, p, 0);
   else
-    hipLaunchKernelGGL(linattn_merge_kernel<false>, dim3((unsigned)bh), blk, 0, s, p);
+    hipLaunchKernelGGL(linattn_merge_kernel<false>, grid2, blk, 0, s, p, nq ? 1 : 0);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const dim3 grid3((unsigned)(bh * ((a.Sq + 127) / 128)));
   if (ea) {
-    if (p.out_f32)
-      hipLaunchKernelGGL((linattn_out_kernel<true, true>), grid3, blk, 0, s, p);
+    if (f32)
+      hipLaunchKernelGGL((linattn_out_kernel<true, true>), grid1, blk, 0, s, p);
     else
-      hipLaunchKernelGGL((linattn_out_kernel<true, false>), grid3, blk, 0, s, p);
+      hipLaunchKernelGGL((linattn_out_kernel<true, false>), grid1, blk, 0, s, p);
   } else {
-    if (p.out_f32)
-      hipLaunchKernelGGL((linattn_out_kernel<false, true>), grid3, blk, 0, s, p);
+    if (f32)
+      hipLaunchKernelGGL((linattn_out_kernel<false, true>), grid1, blk, 0, s, p);
     else
-      hipLaunchKernelGGL((linattn_out_kernel<false, false>), grid3, blk, 0, s, p);
+      hipLaunchKernelGGL((linattn_out_kernel<false, false>), grid1, blk, 0, s, p);
   }
   return hipGetLastError();
 }
