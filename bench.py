@@ -1,6 +1,6 @@
 """Benchmark of the fused attention + per-key score path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--calibrate-copy]
 
 A step is one H2O call (attention forward + column-statistics pass, the two launches behind
 ft_attn_colstats_fwd) on B=1, H=32, S=4096, D=128 fp16 inputs already resident in HBM.  Prints ONE JSON
@@ -22,12 +22,13 @@ if ROOT not in sys.path:
 PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM bytes per launch of the attention kernel at the benchmark shape, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE scaled by a copy kernel of known size (profiles/attn_fwd_h2o_s4096_pmc.txt); None until measured
-ATTN_TRAFFIC_BYTES = None
+# HBM-side bytes per launch of the attention kernel at the benchmark shape, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE) scaled by the readings of a 256 MiB tensor copy in the same run (--calibrate-copy):
+# 78496 x 2 KiB read + 33282 x 1 KiB written (profiles/attn_colstats_h2o_s4096_pmc_traffic.txt)
+ATTN_TRAFFIC_BYTES = 194.84e6
 
 
-def event_time_us(fn, iters, warmup=3):
+def event_time_us(fn, iters, warmup=20):
   import torch
   for _ in range(warmup):
     fn()
@@ -51,7 +52,7 @@ def per_config_table(dev):
   def qkv(B, S, H, D):
     return tuple(torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3))
 
-  def add(name, shape, fn, flops, nbytes, iters=20):
+  def add(name, shape, fn, flops, nbytes, iters=100):
     us = event_time_us(fn, iters)
     tf, gb = flops / us / 1e6, nbytes / us / 1e3
     rows.append({"config": name, "shape": shape, "us": round(us, 1), "tflops": round(tf, 1),
@@ -97,11 +98,14 @@ def cpu_baseline(B, S, H, D, heads):
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
-  ap.add_argument("--steps", type=int, default=50)
-  ap.add_argument("--warmup", type=int, default=10)
+  ap.add_argument("--steps", type=int, default=500)
+  ap.add_argument("--warmup", type=int, default=200)
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
   ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
   ap.add_argument("--cpu-heads", type=int, default=4)
+  ap.add_argument("--calibrate-copy", action="store_true",
+                  help="also run a 256 MiB device-to-device tensor copy a few times: under rocprofv3 --pmc its "
+                       "FETCH_SIZE / WRITE_SIZE readings give the counter unit for the other kernels")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     sys.exit("bench.py: this path runs on ONE GPU (heads/batches shard with no communication); run with --gpus 1")
@@ -122,6 +126,14 @@ def main():
 
   def step():
     return ops.h2o(q, k, v)
+
+  if args.calibrate_copy:
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(5):
+      dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
   for _ in range(args.warmup):
     step()

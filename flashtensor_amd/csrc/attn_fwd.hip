@@ -55,7 +55,12 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   const int BH = p.B * p.H;
   const int nMB = (p.Sq + BM - 1) / BM;
   const int bh = blockIdx.x % BH;
-  const int mb = nMB - 1 - blockIdx.x / BH;  // heaviest (last) query blocks first under the causal mask
+  // Heaviest (last) query blocks of every head first: longest-processing-time order keeps the causal
+  // triangle balanced over the CUs.  Workgroups are dealt round-robin to the 8 XCDs, so with B*H a
+  // multiple of 8 a head stays on one XCD and its K/V are shared through that XCD's L2.  (Walking an XCD
+  // through its heads one at a time cuts the K/V re-reads from 1.6x to 1.1x of the operand size but
+  // loses the balance: measured 15% slower.)
+  const int mb = nMB - 1 - blockIdx.x / BH;
   const int b = bh / p.H, h = bh % p.H;
   const int m0 = mb * BM;
   const int lane = lane_id(), wave = wave_id();
