@@ -11,12 +11,13 @@ LIB_PATH = os.path.join(_HERE, "libflashtensor_hip.so")
 FT_OK, FT_EINVAL, FT_EUNSUPPORTED, FT_ELAUNCH, FT_EWORKSPACE = 0, -1, -2, -3, -4
 FT_F16, FT_BF16, FT_F32 = 0, 1, 2
 FT_CAUSAL, FT_FAST_LOGITS = 1, 2
-FT_OP_ATTN, FT_OP_COLSTATS, FT_OP_KEYFORMER, FT_OP_EA, FT_OP_SIMA = 0, 1, 2, 3, 4
-ABI_VERSION = 1
+FT_OP_ATTN, FT_OP_COLSTATS, FT_OP_KEYFORMER, FT_OP_EA, FT_OP_SIMA, FT_OP_CORM = 0, 1, 2, 3, 4, 5
+ABI_VERSION = 2
 
 # every symbol include/ft_abi.h declares
 EXPORTS = ("ft_abi_version", "ft_last_error", "ft_workspace_bytes", "ft_attn_fwd", "ft_attn_colstats_fwd",
-           "ft_keyformer_fwd", "ft_linattn_fwd", "ft_topk", "ft_noise_exp_fill", "ft_noise_exp_fill_host")
+           "ft_keyformer_fwd", "ft_attn_softcap_fwd", "ft_corm_fwd", "ft_avgpool1d", "ft_linattn_fwd", "ft_topk",
+           "ft_noise_exp_fill", "ft_noise_exp_fill_host")
 
 
 class FtStrides(ctypes.Structure):
@@ -69,6 +70,12 @@ def load():
   lib.ft_attn_colstats_fwd.argtypes = [args_p, f32p, f32p, vp, ctypes.c_size_t, vp]
   lib.ft_keyformer_fwd.restype = ctypes.c_int
   lib.ft_keyformer_fwd.argtypes = [args_p, noise_p, ctypes.c_float, f32p, vp, ctypes.c_size_t, vp]
+  lib.ft_attn_softcap_fwd.restype = ctypes.c_int
+  lib.ft_attn_softcap_fwd.argtypes = [args_p, ctypes.c_float, f32p, vp]
+  lib.ft_corm_fwd.restype = ctypes.c_int
+  lib.ft_corm_fwd.argtypes = [args_p, f32p, ctypes.c_int64, vp, f32p, vp, ctypes.c_size_t, vp]
+  lib.ft_avgpool1d.restype = ctypes.c_int
+  lib.ft_avgpool1d.argtypes = [f32p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, f32p, vp]
   lib.ft_linattn_fwd.restype = ctypes.c_int
   lib.ft_linattn_fwd.argtypes = [args_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, ctypes.c_size_t, vp]
   lib.ft_topk.restype = ctypes.c_int

@@ -23,6 +23,7 @@ hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int ou
 size_t linattn_workspace_bytes(const FtAttnArgs& a, int kind);
 hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* idx, hipStream_t s);
 hipError_t launch_noise_fill(float* dst, int B, int H, int Sq, int Skv, uint64_t seed, hipStream_t s);
+hipError_t launch_avgpool1d(const float* src, int64_t rows, int S, int kernel, float* dst, hipStream_t s);
 }  // namespace ft
 
 namespace {
@@ -192,6 +193,7 @@ size_t ft_workspace_bytes(int op, const FtAttnArgs* a) {
       return 0;
     case FT_OP_COLSTATS:
     case FT_OP_KEYFORMER:
+    case FT_OP_CORM:
       return lse_bytes(a);
     case FT_OP_EA:
     case FT_OP_SIMA:
@@ -274,6 +276,57 @@ int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float
   e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, tensor ? ft::kStatKfTensor : ft::kStatKfSeeded,
                           (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "colstats (keyformer) launch");
+  return FT_OK;
+}
+
+int ft_attn_softcap_fwd(const FtAttnArgs* a, float softcap, float* lse, void* stream) {
+  if (int rc = validate_attn(a, true)) return rc;
+  if (!(softcap > 0.f) || !std::isfinite(softcap)) return fail(FT_EINVAL, "softcap must be positive and finite (got %g)", (double)softcap);
+  const bool emu = !(a->flags & FT_FAST_LOGITS);
+  ft::AttnKernelParams p = attn_params(a, emu);
+  p.lse = lse;
+  p.softcap = softcap;
+  hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, a->flags & FT_CAUSAL, emu, ft::kKfSoftcap, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "attn_fwd (softcap) launch");
+  return FT_OK;
+}
+
+int ft_corm_fwd(const FtAttnArgs* a, const float* corm_mask, int64_t mask_row_stride, uint8_t* corm_score, float* margin,
+                void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = validate_attn(a, true)) return rc;
+  if (!corm_score) return fail(FT_EINVAL, "corm_score pointer is null");
+  if (corm_mask && (mask_row_stride < a->Skv || (reinterpret_cast<uintptr_t>(corm_mask) & 3u)))
+    return fail(FT_EINVAL, "corm_mask needs a contiguous last axis and row stride >= Skv");
+  if (!workspace || workspace_bytes < lse_bytes(a))
+    return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", lse_bytes(a), workspace ? workspace_bytes : (size_t)0);
+  if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(FT_EINVAL, "workspace must be 4-byte aligned");
+  const bool emu = !(a->flags & FT_FAST_LOGITS);
+  const bool causal = a->flags & FT_CAUSAL;
+  float* lse = static_cast<float*>(workspace);
+  ft::AttnKernelParams p = attn_params(a, emu);
+  p.lse = lse;
+  hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, causal, emu, ft::kKfNone, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "attn_fwd launch");
+  ft::ColstatsKernelParams c = col_params(a, emu, lse, margin, nullptr);
+  c.keep = corm_score;
+  if (corm_mask) {
+    c.exp_rand = corm_mask;
+    c.er_sr = mask_row_stride;
+  }
+  e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, corm_mask ? ft::kStatCormTensor : ft::kStatCormRule,
+                          (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "colstats (corm) launch");
+  return FT_OK;
+}
+
+int ft_avgpool1d(const float* src, int64_t rows, int32_t S, int32_t kernel, float* dst, void* stream) {
+  if (!src || !dst) return fail(FT_EINVAL, "src / dst pointer is null");
+  if (src == dst) return fail(FT_EINVAL, "src and dst must not alias");
+  if (rows < 1 || S < 1) return fail(FT_EINVAL, "bad shape rows=%lld S=%d", (long long)rows, S);
+  if (kernel < 1 || (kernel & 1) == 0) return fail(FT_EINVAL, "kernel must be odd and positive (got %d): only then is the output as long as the input", kernel);
+  if (rows > 65535) return fail(FT_EUNSUPPORTED, "too many rows");
+  hipError_t e = ft::launch_avgpool1d(src, rows, S, kernel, dst, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "avgpool1d launch");
   return FT_OK;
 }
 

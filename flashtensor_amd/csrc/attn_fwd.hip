@@ -190,24 +190,32 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   // ---- mask-free fp16 softmax, in two parts so that the rescale branch sits between them.
   // Rounding is monotonic, so the row maximum of the rounded logits is the rounded maximum of the raw
   // accumulators.
-  auto fast_max = [&](const float16v (&s)[2]) {
+  // MASKED (tiles that straddle the diagonal or the end of K): hidden keys are left out of the maximum, so
+  // that a row whose largest visible logit defines the stabiliser gets exp2(0) = 1 for it exactly (row 0
+  // of a causal problem then has the normaliser of the reference, bit for bit).
+  auto fast_max = [&](auto masked_tag, const float16v (&s)[2], int n0) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0 - 4 * g;
+    auto at = [&](int mbk, int r) -> float {
+      if (!MASKED) return s[mbk][r];
+      const int jl = 32 * mbk + 8 * (r >> 2) + (r & 3);
+      return jl > lim ? NEG_INF : s[mbk][r];
+    };
     // four independent chains, then a short tree: the reduction is latency-, not throughput-bound
     float m4[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int mbk = c >> 1, r0 = (c & 1) * 8;
-      m4[c] = max3(s[mbk][r0], s[mbk][r0 + 1], s[mbk][r0 + 2]);
-      m4[c] = max3(m4[c], s[mbk][r0 + 3], s[mbk][r0 + 4]);
-      m4[c] = max3(m4[c], s[mbk][r0 + 5], s[mbk][r0 + 6]);
-      m4[c] = __builtin_fmaxf(m4[c], s[mbk][r0 + 7]);
+      m4[c] = max3(at(mbk, r0), at(mbk, r0 + 1), at(mbk, r0 + 2));
+      m4[c] = max3(m4[c], at(mbk, r0 + 3), at(mbk, r0 + 4));
+      m4[c] = max3(m4[c], at(mbk, r0 + 5), at(mbk, r0 + 6));
+      m4[c] = __builtin_fmaxf(m4[c], at(mbk, r0 + 7));
     }
     float amax = __builtin_fmaxf(max3(m4[0], m4[1], m4[2]), m4[3]);
     amax = __builtin_fmaxf(amax, xchg32(amax));
     rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
   };
-  // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.  The row
-  // maximum above is taken over hidden keys too: any upper bound of the visible logits is a valid
-  // stabiliser, and hidden logits come from the same distribution.
+  // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.
   auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const float neg_m = -m_run;
@@ -268,7 +276,14 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
           if (EMU) {
             x = T::to_float(T::from_float(x));
             x = T::to_float(T::from_float(x * p.logit_mul));
+            if (KF == kKfSoftcap) {  // three 16-bit tensor ops in the reference (cases/kernels/gemma2.py:31-33)
+              x = T::to_float(T::from_float(x / p.softcap));
+              x = T::to_float(T::from_float(tanh_f32(x)));
+              x = T::to_float(T::from_float(x * p.softcap));
+            }
             x *= kLog2e;
+          } else if (KF == kKfSoftcap) {
+            x = p.softcap * tanh_f32(x * (p.logit_mul * (1.f / kLog2e)) / p.softcap) * kLog2e;
           } else {
             x *= p.logit_mul;
           }
@@ -282,7 +297,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       rowmax = fmaxf(rowmax, xchg32(rowmax));
 
       // ---- KeyFormer: running normaliser of softmax((logit + gumbel) / tau), gumbel = -ln(E)
-      if (KF != kKfNone) {
+      if (KF == kKfTensor || KF == kKfSeeded) {
         float z[2][16];
         float zmax = NEG_INF;
 #pragma unroll
@@ -369,7 +384,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     // block, one every few MFMAs.  Issued back to back they fill the texture-address queue (one 1 KB load
     // per 16 cycles per CU) and the wave stalls at issue for about a sixth of the tile time.
     qk_part(s_next, tk_next, std::integral_constant<int, 0>{}, std::integral_constant<int, KSTEPS / 2>{});
-    fast_max(s_cur);
+    fast_max(masked_tag, s_cur, n0);
     if (STAGE) {  // after the rescale branch, so that the loads share a basic block with most of the MFMAs
       stK.issue_full((it + 2) * BN, k_dst);
       stV.issue_full((it + 1) * BN, v_dst);
@@ -483,7 +498,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       }
     if (g == 0 && p.lse) p.lse[(int64_t)bh * p.Sq + qi] = m_run + __builtin_amdgcn_logf(l_run);
   }
-  if (KF != kKfNone) {
+  if (KF == kKfTensor || KF == kKfSeeded) {
     l_kf += xchg32(l_kf);
     if (qi < p.Sq && g == 0) p.lse_kf[(int64_t)bh * p.Sq + qi] = m_kf + __builtin_amdgcn_logf(l_kf);
   }
@@ -507,6 +522,7 @@ static hipError_t launch_td(const AttnKernelParams& p, bool causal, bool emu, in
   FT_CASE(true, true, kKfNone) FT_CASE(true, false, kKfNone) FT_CASE(false, true, kKfNone) FT_CASE(false, false, kKfNone)
   FT_CASE(true, true, kKfTensor) FT_CASE(true, false, kKfTensor) FT_CASE(false, true, kKfTensor) FT_CASE(false, false, kKfTensor)
   FT_CASE(true, true, kKfSeeded) FT_CASE(true, false, kKfSeeded) FT_CASE(false, true, kKfSeeded) FT_CASE(false, false, kKfSeeded)
+  FT_CASE(true, true, kKfSoftcap) FT_CASE(true, false, kKfSoftcap) FT_CASE(false, true, kKfSoftcap) FT_CASE(false, false, kKfSoftcap)
 #undef FT_CASE
   return hipErrorInvalidValue;
 }

@@ -82,4 +82,28 @@ hipError_t launch_noise_fill(float* dst, int B, int H, int Sq, int Skv, uint64_t
   return hipGetLastError();
 }
 
+// Stride-1 window mean along rows of length S with kernel / 2 zeros on both sides, divisor = kernel: the
+// SnapKV smoothing of the per-key scores, F.avg_pool1d(score, kernel, padding = kernel // 2, stride = 1)
+// (cases/kernels/snapkv.py:39).  The window is summed left to right like the library routine.
+__global__ void __launch_bounds__(256) avgpool1d_kernel(const float* __restrict__ src, float* __restrict__ dst, int S, int kernel) {
+  const int64_t row = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= S) return;
+  const float* r = src + row * S;
+  const int pad = kernel / 2;
+  float acc = 0.f;
+  for (int t = -pad; t <= pad; ++t) {
+    const int jj = j + t;
+    if (jj >= 0 && jj < S) acc += r[jj];
+  }
+  dst[row * S + j] = acc / (float)kernel;
+}
+
+hipError_t launch_avgpool1d(const float* src, int64_t rows, int S, int kernel, float* dst, hipStream_t s) {
+  if (rows > 65535) return hipErrorInvalidValue;
+  dim3 grid((unsigned)((S + 255) / 256), (unsigned)rows);
+  hipLaunchKernelGGL(avgpool1d_kernel, grid, dim3(256), 0, s, src, dst, S, kernel);
+  return hipGetLastError();
+}
+
 }  // namespace ft

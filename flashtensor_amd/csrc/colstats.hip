@@ -39,6 +39,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   typedef typename T::vec8 vec8;
   constexpr int TILE_BYTES = BQ * G::RB;
   constexpr bool KFM = (MODE == kStatKfTensor || MODE == kStatKfSeeded);
+  constexpr bool CORM = (MODE == kStatCormRule || MODE == kStatCormTensor);
   constexpr bool kPacked = __is_same(typename T::elem, _Float16) && EMU;  // packed-fp16 rounding chain
   // one LDS object per buffer: reads of one do not wait for the direct-to-LDS loads in flight into the other
   __shared__ __align__(16) char ldsQ0[TILE_BYTES];
@@ -82,7 +83,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
     nk = noise_keys(p.seed, (uint32_t)bh);
     b_j = noise_col(nk, (uint32_t)kj);
   }
-  if (MODE == kStatKfTensor) er_col = p.exp_rand + b * p.er_sb + h * p.er_sh + kj_c;
+  if (MODE == kStatKfTensor || MODE == kStatCormTensor) er_col = p.exp_rand + b * p.er_sb + h * p.er_sh + kj_c;
 
   TileStager<D, BQ, NT, kRowSwizzle> stQ;
   stQ.init(qbase, p.sq.s);
@@ -91,6 +92,12 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   for (int t = 0; t < KSTEPS; ++t) qoff[t] = n * G::RB + (((2 * t + g) ^ G::row_swz(n)) << 4);
 
   float sum[4] = {0.f, 0.f, 0.f, 0.f}, sumsq[4] = {0.f, 0.f, 0.f, 0.f};  // independent chains
+  // CoRM: running maximum over the rows of log2(p / threshold) (rule mode) or p - threshold (tensor mode).
+  // A probability within kCormSlack (relative) of its threshold counts as reaching it: the cases that sit
+  // exactly on the boundary in the reference (p_00 == 1 against 1, equal logits against 1 / (i + 1)) are
+  // kept as they are there, whatever the last bit of the normaliser.
+  constexpr float kCormSlack = 1e-6f;
+  float best[4] = {NEG_INF, NEG_INF, NEG_INF, NEG_INF};
 
   auto stage_q = [&](int t, char* dst) {
     if (t < ntiles) stQ.issue(i_begin + t * BQ, min(BQ, p.Sq - (i_begin + t * BQ)), dst);
@@ -99,7 +106,10 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   auto stage_rows = [&](int t) {
     if (t < ntiles && threadIdx.x < BQ) {
       const int i = i_begin + t * BQ + threadIdx.x;
-      ldsLse[(t & 1) * BQ + threadIdx.x] = i < p.Sq ? -lse_bh[i] : NEG_INF;  // negated: one fma per logit
+      float nl = i < p.Sq ? -lse_bh[i] : NEG_INF;  // negated: one fma per logit
+      // CoRM rule: p_ij >= 1 / (i + 1)  <=>  log2 p_ij + log2(i + 1) >= 0, so no exponential is needed
+      if (MODE == kStatCormRule) nl += __builtin_amdgcn_logf((float)(i + 1));
+      ldsLse[(t & 1) * BQ + threadIdx.x] = nl;
       if (MODE == kStatKfSeeded) ldsRow[(t & 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)i);
     }
   };
@@ -135,7 +145,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
     const int buf = t & 1;
     const int i0 = i_begin + t * BQ;
     float er[2][16];
-    if (MODE == kStatKfTensor) {
+    if (MODE == kStatKfTensor || MODE == kStatCormTensor) {
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
@@ -193,9 +203,17 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
         for (int e = 0; e < 4; ++e) {
           float xv = x[e];
           if (MASKED) xv = (il0 + e < lim) ? NEG_INF : xv;
-          const float pr = __builtin_amdgcn_exp2f(xv);
-          sum[e] += pr;
-          if (MODE == kStatSumSq) sumsq[e] = __builtin_fmaf(pr, pr, sumsq[e]);
+          if (MODE == kStatCormRule) {
+            best[e] = fmaxf(best[e], xv);
+          } else {
+            const float pr = __builtin_amdgcn_exp2f(xv);
+            if (MODE == kStatCormTensor) {
+              best[e] = fmaxf(best[e], pr - er[mbk][4 * q4 + e] * (1.f - kCormSlack));
+            } else {
+              sum[e] += pr;
+              if (MODE == kStatSumSq) sumsq[e] = __builtin_fmaf(pr, pr, sumsq[e]);
+            }
+          }
         }
       }
   };
@@ -268,10 +286,17 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   tot += xchg32(tot);
   float totsq = (sumsq[0] + sumsq[1]) + (sumsq[2] + sumsq[3]);
   if (MODE == kStatSumSq) totsq += xchg32(totsq);
+  float top = fmaxf(fmaxf(best[0], best[1]), fmaxf(best[2], best[3]));
+  if (CORM) top = fmaxf(top, xchg32(top));
   if (g == 0 && kj < p.Skv) {
     const int64_t idx = (int64_t)bh * p.Skv + kj;
-    p.colsum[idx] = tot;
-    if (MODE == kStatSumSq) p.colsumsq[idx] = totsq;
+    if (CORM) {
+      p.keep[idx] = top >= (MODE == kStatCormRule ? -kCormSlack * kLog2e : 0.f) ? 1 : 0;
+      if (p.colsum) p.colsum[idx] = top;  // optional: distance from the decision boundary
+    } else {
+      p.colsum[idx] = tot;
+      if (MODE == kStatSumSq) p.colsumsq[idx] = totsq;
+    }
   }
 }
 
@@ -289,7 +314,9 @@ template <typename T, int D>
 static hipError_t launch_td(const ColstatsKernelParams& p, bool causal, bool emu, int mode, hipStream_t s) {
 #define FT_CASE(C, E, M) \
   if (causal == C && emu == E && mode == M) return launch_one<T, D, C, E, M>(p, s);
-#define FT_MODES(C, E) FT_CASE(C, E, kStatSum) FT_CASE(C, E, kStatSumSq) FT_CASE(C, E, kStatKfTensor) FT_CASE(C, E, kStatKfSeeded)
+#define FT_MODES(C, E)                                                                                       \
+  FT_CASE(C, E, kStatSum) FT_CASE(C, E, kStatSumSq) FT_CASE(C, E, kStatKfTensor) FT_CASE(C, E, kStatKfSeeded) \
+  FT_CASE(C, E, kStatCormRule) FT_CASE(C, E, kStatCormTensor)
   FT_MODES(true, true) FT_MODES(true, false) FT_MODES(false, true) FT_MODES(false, false)
 #undef FT_MODES
 #undef FT_CASE

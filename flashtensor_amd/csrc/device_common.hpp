@@ -82,6 +82,17 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return r;
 }
 
+// tanh to fp32 accuracy without a hardware instruction: odd polynomial where 1 - 2 / (e^2y + 1) would
+// cancel (|y| < 0.25, truncation error < 4e-7 relative), the exponential form elsewhere.
+__device__ __forceinline__ float tanh_f32(float y) {
+  const float a = __builtin_fabsf(y);
+  const float y2 = y * y;
+  const float poly = y * (1.f + y2 * (-1.f / 3.f + y2 * (2.f / 15.f + y2 * (-17.f / 315.f + y2 * (62.f / 2835.f)))));
+  const float e = __builtin_amdgcn_exp2f(a * (2.f * kLog2e));
+  const float big = __builtin_copysignf(1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f), y);
+  return a < 0.25f ? poly : big;
+}
+
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
 // ---------------------------------------------------------------------------------------------------

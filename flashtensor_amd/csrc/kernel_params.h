@@ -24,6 +24,7 @@ struct AttnKernelParams {
   int off;          // Skv - Sq: query i sees keys j <= i + off when causal
   float logit_mul;  // reference rounding: f16(f16(acc) * logit_mul) == f16(f16(acc) / sqrt(D)); fast: log2e / sqrt(D)
   float inv_tau;
+  float softcap;    // kKfSoftcap: logits become softcap * tanh(logit / softcap)
 };
 
 struct ColstatsKernelParams {
@@ -33,7 +34,8 @@ struct ColstatsKernelParams {
   const float* lse;  // [B,H,Sq] normaliser of the distribution being summed
   float* colsum;     // [B,H,Skv]
   float* colsumsq;   // [B,H,Skv] or null
-  const float* exp_rand;
+  uint8_t* keep;     // [B,H,Skv] CoRM modes: 1 where some row's probability reaches its threshold
+  const float* exp_rand;  // KeyFormer noise [B,H,Sq,Skv]; CoRM tensor mode: thresholds [Sq,Skv] (er_sb = er_sh = 0)
   int64_t er_sb, er_sh, er_sr;
   uint64_t seed;
   int B, H, Sq, Skv;
@@ -42,7 +44,9 @@ struct ColstatsKernelParams {
   float inv_tau;
 };
 
-enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2 };
-enum StatMode { kStatSum = 0, kStatSumSq = 1, kStatKfTensor = 2, kStatKfSeeded = 3 };
+// what happens to a logit between the scaled QK^T and the softmax of the attention pass
+enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2, kKfSoftcap = 3 };
+// kStatCormRule: thresholds 1 / (i + 1) per query row i; kStatCormTensor: thresholds read from a tensor
+enum StatMode { kStatSum = 0, kStatSumSq = 1, kStatKfTensor = 2, kStatKfSeeded = 3, kStatCormRule = 4, kStatCormTensor = 5 };
 
 }  // namespace ft

@@ -90,6 +90,46 @@ class KeyFormer(_Case):
     return ret
 
 
+class SnapKV(_Case):
+  """cases/kernels/snapkv.py: (out, snapkv_score); kernel_size defaults to 5 as snapkv.py:8."""
+  output = ["out", "snapkv_score"]
+
+  def __init__(self, kernel_size=5, kv_head_num=32, head_num=32, head_dim=128):
+    super().__init__(kv_head_num, head_num, head_dim)
+    self.kernel_size = kernel_size
+
+  def forward(self, q, k, v):
+    return ops.snapkv(q, k, v, kernel_size=self.kernel_size)
+
+
+class Corm(_Case):
+  """cases/kernels/corm.py: (out, corm_score bool).  Passing corm_mask=None to forward applies the
+  prepare() thresholds 1 / (i + 1) without materialising them."""
+  output = ["out", "corm_score"]
+
+  def forward(self, q, k, v, corm_mask=None):
+    return ops.corm(q, k, v, corm_mask)
+
+  def prepare(self, batch_size=1, q_len=4096, kv_len=4096, dtype=torch.float16, device=None):
+    ret = super().prepare(batch_size, q_len, kv_len, dtype, device)
+    dev = ret["input"]["q"].device
+    rows = torch.arange(1, q_len + 1, dtype=torch.float32, device=dev).unsqueeze(1)
+    ret["input"]["corm_mask"] = torch.ones(q_len, kv_len, dtype=torch.float32, device=dev) / rows  # corm.py:47-49
+    return ret
+
+
+class Gemma2(_Case):
+  """cases/kernels/gemma2.py: out, logits soft-capped at logit_softcapping (default 50, gemma2.py:8)."""
+  output = ["out"]
+
+  def __init__(self, logit_softcapping=50.0, kv_head_num=32, head_num=32, head_dim=128):
+    super().__init__(kv_head_num, head_num, head_dim)
+    self.logit_softcapping = logit_softcapping
+
+  def forward(self, q, k, v):
+    return ops.gemma2(q, k, v, softcap=self.logit_softcapping)
+
+
 class EA(_Case):
   """Attention core of bench/ea.mlir:13-17 on [B,S,H,D] tensors."""
   output = ["out"]
@@ -115,7 +155,8 @@ class SimA(EA):
     return ops.sima(q, k, v, normalize_q=self.normalize_q)
 
 
-CASES = {"attn": Attn, "h2o": H2O, "kf": KeyFormer, "roco": RoCo, "ea": EA, "sima": SimA}
+CASES = {"attn": Attn, "h2o": H2O, "kf": KeyFormer, "roco": RoCo, "snapkv": SnapKV, "corm": Corm, "gemma2": Gemma2,
+         "ea": EA, "sima": SimA}
 
 
 def get_model(name="attn", **kw):

@@ -123,6 +123,55 @@ def keyformer(q, k, v, exp_rand=None, tau=1.5, seed=0, causal=True, fast_logits=
   return out, score
 
 
+def snapkv(q, k, v, kernel_size=5, causal=True, fast_logits=False):
+  """SnapKV.forward (cases/kernels/snapkv.py:19-43) -> (out, snapkv_score [B,H,Skv] fp32): the H2O column
+  sums smoothed by a stride-1 average pool of odd width `kernel_size` over the key axis."""
+  out, score = _colstats(q, k, v, False, causal, fast_logits)
+  lib = _lib.load()
+  B, H, Skv = score.shape
+  pooled = torch.empty_like(score)
+  _lib.check(lib.ft_avgpool1d(score.data_ptr(), B * H, Skv, int(kernel_size), pooled.data_ptr(), _stream(q)))
+  return out, pooled
+
+
+def corm(q, k, v, corm_mask=None, causal=True, fast_logits=False, return_margin=False):
+  """Corm.forward (cases/kernels/corm.py:18-40) -> (out, corm_score [B,H,Skv] bool): key j is kept when some
+  query row gives it a probability >= corm_mask[i, j].  corm_mask [Sq,Skv] fp32 is the reference's input;
+  None applies its prepare() recipe 1 / (i + 1) (corm.py:47-49) without reading a tensor."""
+  q, k, v = _prep(q, k, v)
+  lib = _lib.load()
+  B, Sq, H, D = q.shape
+  Skv = k.shape[1]
+  mask_ptr, mask_stride = None, 0
+  if corm_mask is not None:
+    if tuple(corm_mask.shape) != (Sq, Skv):
+      raise RuntimeError(f"arg 3 need shape {(Sq, Skv)} but got {tuple(corm_mask.shape)}")
+    if corm_mask.dtype != torch.float32 or corm_mask.device != q.device:
+      raise RuntimeError(f"arg 3 need dtype torch.float32 on {q.device} but got {corm_mask.dtype} on {corm_mask.device}")
+    corm_mask = _dense_last(corm_mask)
+    mask_ptr, mask_stride = corm_mask.data_ptr(), corm_mask.stride(0)
+  out = torch.empty_like(q, memory_format=torch.contiguous_format)
+  keep = torch.empty(B, H, Skv, dtype=torch.uint8, device=q.device)
+  margin = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device) if return_margin else None
+  a = _args(q, k, v, out, _flags(causal, fast_logits))
+  nbytes = lib.ft_workspace_bytes(_lib.FT_OP_CORM, ctypes.byref(a))
+  ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+  _lib.check(lib.ft_corm_fwd(ctypes.byref(a), mask_ptr, mask_stride, keep.data_ptr(),
+                             margin.data_ptr() if return_margin else None, ws.data_ptr(), nbytes, _stream(q)))
+  keep = keep.view(torch.bool)
+  return (out, keep, margin) if return_margin else (out, keep)
+
+
+def gemma2(q, k, v, softcap=50.0, causal=True, fast_logits=False):
+  """Gemma2.forward (cases/kernels/gemma2.py:19-39): attention with logits softcap * tanh(logit / softcap)."""
+  q, k, v = _prep(q, k, v)
+  lib = _lib.load()
+  out = torch.empty_like(q, memory_format=torch.contiguous_format)
+  a = _args(q, k, v, out, _flags(causal, fast_logits))
+  _lib.check(lib.ft_attn_softcap_fwd(ctypes.byref(a), float(softcap), None, _stream(q)))
+  return out
+
+
 def _linattn(q, k, v, kind, normalize_q, out_dtype):
   q, k, v = _prep(q, k, v)
   lib = _lib.load()

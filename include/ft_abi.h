@@ -12,7 +12,7 @@
  *   results and launches the fused Triton kernel (lib/Translate/to_triton.cpp:529-638, device kernel
  *   :480-527), and the TensorRT closure used by the harnesses
  *   (python/asuka/backend/tensorrt/builder.py:73-151), for the workloads defined in
- *   cases/kernels/{attn,h2o,kf,roco}.py and bench/{ea,sima}.mlir.
+ *   cases/kernels/{attn,h2o,kf,roco,snapkv,corm,gemma2}.py and bench/{ea,sima}.mlir.
  */
 #ifndef FT_ABI_H
 #define FT_ABI_H
@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FT_ABI_VERSION 1
+#define FT_ABI_VERSION 2
 
 enum FtStatus {
   FT_OK = 0,
@@ -42,7 +42,7 @@ enum FtFlags {
                           of the logits (cases/kernels/attn.py:29); faster, ~1e-3 relative on probabilities */
 };
 
-enum FtOp { FT_OP_ATTN = 0, FT_OP_COLSTATS = 1, FT_OP_KEYFORMER = 2, FT_OP_EA = 3, FT_OP_SIMA = 4 };
+enum FtOp { FT_OP_ATTN = 0, FT_OP_COLSTATS = 1, FT_OP_KEYFORMER = 2, FT_OP_EA = 3, FT_OP_SIMA = 4, FT_OP_CORM = 5 };
 
 /* Element strides of a logical [B, S, H, D] tensor; the D axis must be contiguous (stride 1). */
 typedef struct FtStrides {
@@ -90,6 +90,25 @@ int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, vo
  * gumbel = -log(exp_rand).  kf_score: [B,H,Skv] fp32. */
 int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float* kf_score, void* workspace,
                      size_t workspace_bytes, void* stream);
+
+/* Gemma2.forward (cases/kernels/gemma2.py:19-39): attention whose scaled logits pass through
+ * softcap * tanh(logit / softcap) (three 16-bit tensor ops in the reference, :31-33) before the mask and
+ * the softmax.  lse: optional [B,H,Sq] fp32 as for ft_attn_fwd. */
+int ft_attn_softcap_fwd(const FtAttnArgs* a, float softcap, float* lse, void* stream);
+
+/* Corm.forward (cases/kernels/corm.py:18-40): attention + corm_score[b,h,j] = any_i(probs[b,h,i,j] >=
+ * corm_mask[i,j]) as uint8 [B,H,Skv].  corm_mask: fp32 [Sq,Skv] with the given row stride, thresholds > 0
+ * (pairs hidden by the causal mask are not compared); NULL = the reference's own recipe 1 / (i + 1)
+ * (corm.py:47-49), evaluated in the log domain without reading a tensor.  A probability within 1e-6
+ * (relative) of its threshold counts as reaching it, so the reference's exact ties (p_00 = 1 against 1) are kept.
+ * margin: optional [B,H,Skv] fp32 distance from the boundary: max_i log2(p_ij (i + 1)) for the recipe,
+ * max_i (p_ij - (1 - 1e-6) mask_ij) for a tensor. */
+int ft_corm_fwd(const FtAttnArgs* a, const float* corm_mask, int64_t mask_row_stride, uint8_t* corm_score, float* margin,
+                void* workspace, size_t workspace_bytes, void* stream);
+
+/* SnapKV's smoothing of the per-key scores (cases/kernels/snapkv.py:39): dst[r, j] = (1 / kernel) * sum of
+ * src[r, j - kernel/2 .. j + kernel/2] with zeros outside the row, kernel odd; src, dst: [rows, S] fp32. */
+int ft_avgpool1d(const float* src, int64_t rows, int32_t S, int32_t kernel, float* dst, void* stream);
 
 /* Linear attention cores of bench/ea.mlir:13-17 (kind = FT_OP_EA) and bench/sima.mlir:13-17 (FT_OP_SIMA):
  * O = f(Q) (g(K)^T V).  normalize_q applies SimA's L1 normalisation to Q as well (ignored for EA).

@@ -17,6 +17,14 @@ How each function is pinned (tests/test_oracle_pins.py, tests/test_oracle_golden
                      form; sum_j == Sq; fp64 brute force with random noise.
   ea_forward         V == c -> O == c; Q == K == 0 -> O = mean_s V; fp64 brute force.
   sima_forward       sum_s |Qhat| == 1; scale invariance in Q and K; fp64 brute force.
+  snapkv_forward     kernel_size == 1 -> the H2O score; explicit zero-padded window loop in numpy on
+                     top of the fp64 brute-force column sums; interior windows of a constant score.
+  corm_forward       key 0 is always kept (p_00 == 1 >= 1); q == 0 -> p_ij == 1/(i+1) exactly -> every key
+                     kept; an all-ones mask keeps exactly the keys some row attends to with p == 1; fp64
+                     brute force away from the decision boundary (corm_margin).
+  gemma2_forward     softcap = 512 (a power of two, tanh(y) == y in fp16 for the tiny y) -> attn_forward
+                     up to last-bit flips; tiny softcap -> logits ~ 0 -> prefix means of V; fp64 brute
+                     force at caps 50 and 2.
 The reference holds no golden vectors or tests for this path, so none can be checked against; no
 function of this file is "parity unpinned".
 """
@@ -84,6 +92,59 @@ def keyformer_forward(q, k, v, exp_rand, tau=1.5):
   kf_score = F.softmax(kf_score.float(), dim=-1)
   kf_score = kf_score.sum(dim=2)
   return out, kf_score.view(q.shape[0], q.shape[2], k.shape[1])
+
+
+def snapkv_forward(q, k, v, kernel_size=5):
+  """SnapKV, cases/kernels/snapkv.py:19-43 (kernel_size default :8): attention + the per-key column sum
+  of the probabilities smoothed by a stride-1 average pool over keys (zero padding of kernel_size // 2,
+  padded positions counted in the divisor: F.avg_pool1d defaults)."""
+  _, probs = _masked_scores_probs(q, k)
+  out = _out(probs, q, v)
+  snapkv_score = probs.sum(dim=2)
+  snapkv_score = F.avg_pool1d(snapkv_score, kernel_size=kernel_size, padding=kernel_size // 2, stride=1)
+  return out, snapkv_score.view(q.shape[0], q.shape[2], k.shape[1])
+
+
+def corm_mask_rule(q_len, kv_len):
+  """Threshold recipe of Corm.prepare (cases/kernels/corm.py:47-49): row i holds 1 / (i + 1), fp32."""
+  rows = torch.arange(1, q_len + 1, dtype=torch.float32).unsqueeze(1)
+  return torch.ones(q_len, kv_len, dtype=torch.float32) / rows
+
+
+def corm_forward(q, k, v, corm_mask):
+  """CoRM, cases/kernels/corm.py:18-40: attention + corm_score[b,h,j] = any_i(probs[b,h,i,j] >=
+  corm_mask[i,j]) (bool [B,H,Skv]); corm_mask is fp32 [Sq,Skv]."""
+  _, probs = _masked_scores_probs(q, k)
+  out = _out(probs, q, v)
+  corm_score = probs >= corm_mask
+  corm_score = corm_score.any(dim=2)
+  return out, corm_score.view(q.shape[0], q.shape[2], k.shape[1])
+
+
+def corm_margin(q, k, corm_mask):
+  """max_i probs[b,h,i,j] / corm_mask[i,j] ([B,H,Skv] fp32): corm_score is True iff this is >= 1; its
+  distance from 1 tells how far a key is from the decision boundary (used for the comparison rule of
+  the parity tests, not part of the reference)."""
+  _, probs = _masked_scores_probs(q, k)
+  return (probs / corm_mask).amax(dim=2)
+
+
+def gemma2_forward(q, k, v, softcap=50.0):
+  """Gemma2 soft-capped attention, cases/kernels/gemma2.py:19-39 (logit_softcapping default :8): the
+  fp16 scores are divided by the cap, passed through tanh and multiplied by the cap again, each step an
+  fp16 tensor op, before the mask and the fp32 softmax."""
+  q_len, kv_len = q.shape[1], k.shape[1]
+  mask = torch.full((1, 1, q_len, kv_len), -torch.inf, device=q.device, dtype=q.dtype)
+  mask = torch.triu(mask, diagonal=kv_len - q_len + 1)
+  qt = q.transpose(1, 2)
+  kt = k.transpose(1, 2)
+  scores = torch.matmul(qt, kt.transpose(-2, -1)) / math.sqrt(q.shape[3])
+  scores /= softcap
+  scores = torch.tanh(scores)
+  scores *= softcap
+  scores += mask
+  probs = F.softmax(scores.float(), dim=-1)
+  return _out(probs, q, v)
 
 
 def ea_forward(q, k, v):

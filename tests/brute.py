@@ -60,3 +60,50 @@ def sima(q, k, v, normalize_q=True):
       qh = Q / np.abs(Q).sum(axis=0, keepdims=True) if normalize_q else Q
       O[b, :, h] = qh @ (kh.T @ V)
   return O
+
+
+def avg_pool_same(x, kernel):
+  """Stride-1 window mean over the last axis with kernel // 2 zeros on both sides, divisor = kernel."""
+  x = np.asarray(x, dtype=np.float64)
+  pad = kernel // 2
+  out = np.zeros_like(x)
+  n = x.shape[-1]
+  for j in range(n):
+    acc = 0.0
+    for t in range(-pad, pad + 1):
+      if 0 <= j + t < n:
+        acc = acc + x[..., j + t]
+    out[..., j] = acc / kernel
+  return out
+
+
+def corm_ratio(q, k, thr):
+  """max over query rows of p_ij / thr_ij, [B,H,Skv] float64 (thr: [Sq,Skv])."""
+  q, k = (t.numpy() if hasattr(t, "numpy") else t for t in (q, k))
+  thr = thr.numpy().astype(np.float64) if hasattr(thr, "numpy") else thr
+  B, Sq, H, _ = q.shape
+  out = np.zeros((B, H, k.shape[1]))
+  for b in range(B):
+    for h in range(H):
+      _, p = _probs(q, k, b, h)
+      out[b, h] = (p / thr).max(axis=0)
+  return out
+
+
+def softcap_attention(q, k, v, cap):
+  """O of attention whose scaled logits are replaced by cap * tanh(logit / cap), [B,Sq,H,D] float64."""
+  q, k, v = (t.numpy() if hasattr(t, "numpy") else t for t in (q, k, v))
+  B, Sq, H, D = q.shape
+  Skv = k.shape[1]
+  O = np.zeros((B, Sq, H, D))
+  for b in range(B):
+    for h in range(H):
+      s = q[b, :, h, :].astype(np.float64) @ k[b, :, h, :].astype(np.float64).T / np.sqrt(D)
+      s = cap * np.tanh(s / cap)
+      for i in range(Sq):
+        for j in range(Skv):
+          if j > i + (Skv - Sq):
+            s[i, j] = -np.inf
+      e = np.exp(s - s.max(axis=1, keepdims=True))
+      O[b, :, h, :] = (e / e.sum(axis=1, keepdims=True)) @ v[b, :, h, :].astype(np.float64)
+  return O

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(lib):
   assert declared == sorted(_lib.EXPORTS)
   for name in declared:
     assert getattr(lib, name) is not None
-  assert lib.ft_abi_version() == 1
+  assert lib.ft_abi_version() == 2 == _lib.ABI_VERSION
 
 
 def _args(**over):
@@ -75,6 +75,26 @@ def test_colstats_and_keyformer_argument_checks(lib):
   assert lib.ft_keyformer_fwd(ctypes.byref(a), ctypes.byref(noise), 1.0, None, 0x5000, need, None) == _lib.FT_EINVAL
 
 
+def test_softcap_corm_and_avgpool_argument_checks(lib):
+  a = _args()
+  assert lib.ft_attn_softcap_fwd(ctypes.byref(a), 0.0, None, None) == _lib.FT_EINVAL
+  assert "softcap" in lib.ft_last_error().decode()
+  assert lib.ft_attn_softcap_fwd(ctypes.byref(a), float("inf"), None, None) == _lib.FT_EINVAL
+  assert lib.ft_attn_softcap_fwd(ctypes.byref(_args(D=96)), 50.0, None, None) == _lib.FT_EUNSUPPORTED
+  need = lib.ft_workspace_bytes(_lib.FT_OP_CORM, ctypes.byref(a))
+  assert need == 1 * 2 * 8 * 4
+  assert lib.ft_corm_fwd(ctypes.byref(a), None, 0, None, None, 0x5000, need, None) == _lib.FT_EINVAL
+  assert "corm_score" in lib.ft_last_error().decode()
+  assert lib.ft_corm_fwd(ctypes.byref(a), 0x7000, 4, 0x6000, None, 0x5000, need, None) == _lib.FT_EINVAL  # row stride < Skv
+  assert "corm_mask" in lib.ft_last_error().decode()
+  assert lib.ft_corm_fwd(ctypes.byref(a), None, 0, 0x6000, None, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
+  assert lib.ft_avgpool1d(None, 1, 8, 5, 0x2000, None) == _lib.FT_EINVAL
+  assert lib.ft_avgpool1d(0x1000, 1, 8, 4, 0x2000, None) == _lib.FT_EINVAL
+  assert "odd" in lib.ft_last_error().decode()
+  assert lib.ft_avgpool1d(0x1000, 1, 8, 5, 0x1000, None) == _lib.FT_EINVAL
+  assert lib.ft_avgpool1d(0x1000, 0, 8, 5, 0x2000, None) == _lib.FT_EINVAL
+
+
 def test_linattn_and_topk_argument_checks(lib):
   st = FtStrides(64 * 2 * 64, 2 * 64, 64)
   a = _args(D=64, Sq=64, Skv=64, sq=st, sk=st, sv=st, so=st, flags=0)
@@ -109,7 +129,8 @@ def test_operator_layer_validates_like_the_reference_backend():
   f = ft.HipBuilder("h2o").build_callable()
   with pytest.raises(RuntimeError, match="arg 0 need shape"):
     f(torch.zeros(1, 8, 2, 64, dtype=torch.float16), q, q)
-  assert sorted(ft.CASES) == ["attn", "ea", "h2o", "kf", "roco", "sima"]
+  assert sorted(ft.CASES) == ["attn", "corm", "ea", "gemma2", "h2o", "kf", "roco", "sima", "snapkv"]
+  assert ft.get_model("snapkv").kernel_size == 5 and ft.get_model("gemma2").logit_softcapping == 50.0
   assert ft.get_model("kf").tau == 1.5 and ft.get_model("h2o").prepare.__doc__
 
 

@@ -240,6 +240,114 @@ def test_ea_sima_properties(gpu):
   assert torch.allclose(a, b, rtol=1e-4, atol=1e-9)
 
 
+# ------------------------------------------------------------------ SnapKV, CoRM, Gemma2 (the other cases of the zoo)
+
+NEXT_SMALL = [(1, 128, 2, 128, 0), (2, 200, 3, 128, 2), (1, 333, 2, 64, 5), (1, 1, 2, 64, 4), (1, 700, 2, 128, 7)]
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", NEXT_SMALL)
+def test_snapkv_small(gpu, B, S, H, D, seed):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  ref_o, ref_s = oracle.snapkv_forward(q, k, v)
+  out, s = ops.snapkv(qd, kd, vd)
+  check_o(out, ref_o); check_score(s, ref_s)
+  for ks in (1, 3, 9):
+    _, sk = ops.snapkv(qd, kd, vd, kernel_size=ks)
+    check_score(sk, oracle.snapkv_forward(q, k, v, kernel_size=ks)[1])
+  assert torch.equal(ops.snapkv(qd, kd, vd, kernel_size=1)[1], ops.h2o(qd, kd, vd)[1])  # a window of one is the identity
+  with pytest.raises(ValueError, match="odd"):
+    ops.snapkv(qd, kd, vd, kernel_size=4)
+
+
+def check_corm(keep, ratio, tol=1e-3):
+  """keep: GPU result; ratio = max_i p_ij / threshold_ij from the oracle: the decision must agree wherever
+  it is not within `tol` (relative) of the boundary, and nearly all keys must be that clear."""
+  keep = keep.cpu()
+  clear = (ratio - 1).abs() > tol
+  assert clear.numel() < 64 or clear.float().mean().item() > 0.97
+  assert torch.equal(keep[clear], (ratio >= 1)[clear]), f"{(keep[clear] != (ratio >= 1)[clear]).sum().item()} clear keys differ"
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", NEXT_SMALL)
+def test_corm_small(gpu, B, S, H, D, seed):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  rule = oracle.corm_mask_rule(S, S)
+  ref_o, ref_keep = oracle.corm_forward(q, k, v, rule)
+  ratio = oracle.corm_margin(q, k, rule)
+  out, keep, margin = ops.corm(qd, kd, vd, return_margin=True)             # recipe thresholds, no tensor read
+  assert keep.dtype == torch.bool and keep.shape == ref_keep.shape
+  check_o(out, ref_o); check_corm(keep, ratio)
+  assert torch.equal(keep, margin >= -1.5e-6)
+  assert keep[..., 0].all()                                               # p_00 == 1 >= 1
+  # the log-domain margin is log2 of the oracle's ratio
+  fin = ratio > 0
+  assert torch.allclose(margin.cpu()[fin], ratio[fin].log2(), atol=2e-3)
+  out_t, keep_t = ops.corm(qd, kd, vd, rule.to(gpu))                       # the same thresholds as the reference's input tensor
+  check_corm(keep_t, ratio)
+  assert (keep_t != keep).float().mean().item() < 0.01
+  # arbitrary positive thresholds, strided rows
+  g = torch.Generator().manual_seed(seed)
+  wide = torch.rand(S, S + 8, generator=g) * 0.2 + 1e-3
+  thr = wide[:, :S]
+  check_corm(ops.corm(qd, kd, vd, wide.to(gpu)[:, :S])[1], oracle.corm_margin(q, k, thr))
+  # all-ones thresholds keep only key 0
+  k1 = ops.corm(qd, kd, vd, torch.ones(S, S, device=gpu))[1]
+  assert k1[..., 0].all() and not k1[..., 1:].any()
+
+
+def test_corm_zero_queries_keep_every_key(gpu):
+  # p_ij == 1/(i+1) exactly: every decision sits on the boundary, which the >= keeps
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 256, 2, 128, seed=3)
+  _, keep, margin = ops.corm(torch.zeros_like(qd), kd, vd, return_margin=True)
+  assert margin.abs().max().item() < 1e-5
+  assert keep.all()                              # ties count as reached, as in the reference
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", NEXT_SMALL)
+def test_gemma2_small(gpu, B, S, H, D, seed):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  check_o(ops.gemma2(qd, kd, vd), oracle.gemma2_forward(q, k, v))
+  for cap in (2.0, 0.5, 512.0):
+    check_o(ops.gemma2(qd, kd, vd, softcap=cap), oracle.gemma2_forward(q, k, v, softcap=cap))
+  # larger logits, where the cap bends them: 4x the scale puts |logit| up to ~20 against a cap of 8
+  check_o(ops.gemma2(qd * 2, kd * 2, vd, softcap=8.0), oracle.gemma2_forward(q * 2, k * 2, v, softcap=8.0))
+  check_o(ops.gemma2(qd, kd, vd, fast_logits=True), oracle.gemma2_forward(q, k, v), abs_tol=2e-2, tight=1e-2)
+  with pytest.raises(ValueError, match="softcap"):
+    ops.gemma2(qd, kd, vd, softcap=0.0)
+
+
+def test_gemma2_bf16_and_noncausal(gpu):
+  q, k, v = oracle.prepare_inputs(1, 192, 2, 128, seed=9, dtype=torch.bfloat16)
+  out = ops.gemma2(q.to(gpu), k.to(gpu), v.to(gpu), softcap=5.0)
+  ref = oracle.gemma2_forward(q, k, v, softcap=5.0)
+  assert (out.float().cpu() - ref.float()).abs().max().item() <= 6e-2
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 160, 2, 64, seed=10)
+  full = ops.gemma2(qd, kd, vd, softcap=3.0, causal=False)
+  assert torch.isfinite(full).all()
+  # without a mask row i of the causal result for the last query equals the full result's last row
+  assert torch.allclose(full[:, -1].float(), ops.gemma2(qd, kd, vd, softcap=3.0)[:, -1].float(), atol=2e-3)
+
+
+def test_next_cases_at_reference_default_shape(gpu):
+  """B=1 H=32 S=4096 D=128, the prepare() defaults of snapkv.py / corm.py / gemma2.py; oracle on 4 heads."""
+  S, HS = 4096, 4
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, 32, 128, seed=0)
+  qs, ks, vs = (t[:, :, :HS].contiguous() for t in (q, k, v))
+  ref_o, ref_s = oracle.snapkv_forward(qs, ks, vs)
+  out, s = ops.snapkv(qd, kd, vd)
+  check_o(out[:, :, :HS], ref_o); check_score(s[:, :HS], ref_s)
+  h = ops.h2o(qd, kd, vd)[1]
+  assert abs(s.sum().item() * 5 - (5 * h.sum().item() - (2 * h[..., 0] + h[..., 1] + h[..., -2] + 2 * h[..., -1]).sum().item())) < 1e-2 * S
+  rule = oracle.corm_mask_rule(S, S)
+  out_c, keep = ops.corm(qd, kd, vd)
+  check_corm(keep[:, :HS], oracle.corm_margin(qs, ks, rule))
+  assert torch.equal(out_c, out)
+  assert keep[..., 0].all() and (~keep).any()        # only some of the last keys of a head are dropped
+  check_o(ops.gemma2(qd, kd, vd)[:, :, :HS], oracle.gemma2_forward(qs, ks, vs))
+  f = ft.HipBuilder("snapkv").build_callable()
+  assert torch.equal(f(qd, kd, vd)[1], s)
+
+
 # ------------------------------------------------------------------ the five measured configurations
 
 def test_config1_attn_b1_h32_s1024_d128(gpu):

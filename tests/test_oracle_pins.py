@@ -244,3 +244,72 @@ def test_lowbias32_known_answers():
   got = oracle.lowbias32(np.array(xs, dtype=np.uint64))
   assert [int(g) for g in got] == [ref(x) for x in xs]
   assert int(oracle.lowbias32(0)) == 0 and len(set(int(g) for g in got)) == len(xs)
+
+
+# ------------------------------------------------------------------ SnapKV, CoRM, Gemma2
+
+def test_snapkv_pool_closed_forms_and_brute_force():
+  q, k, v = _inputs(S=48, H=2, D=64, seed=11)
+  out_h, score_h = oracle.h2o_forward(q, k, v)
+  out1, s1 = oracle.snapkv_forward(q, k, v, kernel_size=1)
+  assert torch.equal(out1, out_h) and torch.equal(s1, score_h)           # a window of one is the identity
+  out5, s5 = oracle.snapkv_forward(q, k, v)                               # reference default: 5
+  assert torch.equal(out5, out_h) and s5.shape == score_h.shape
+  _, cs, _, _ = brute.attention_stats(q, k, v)
+  np.testing.assert_allclose(s5.numpy(), brute.avg_pool_same(cs, 5), rtol=2e-3, atol=1e-6)
+  # edges: the first output averages only three real entries but still divides by five
+  np.testing.assert_allclose(s5[..., 0].numpy(), (cs[..., 0] + cs[..., 1] + cs[..., 2]) / 5, rtol=2e-3)
+  # q == 0: score_j = H_S - H_j, smooth, so interior windows sit between their neighbours' extremes
+  z = torch.zeros_like(q)
+  _, sz = oracle.snapkv_forward(z, k, v, kernel_size=3)
+  _, hz = oracle.h2o_forward(z, k, v)
+  mid = (hz[..., :-2] + hz[..., 1:-1] + hz[..., 2:]) / 3
+  np.testing.assert_allclose(sz[..., 1:-1].numpy(), mid.numpy(), rtol=1e-5)
+
+
+def test_corm_closed_forms_and_brute_force():
+  S = 40
+  q, k, v = _inputs(S=S, H=2, D=64, seed=12)
+  rule = oracle.corm_mask_rule(S, S)
+  assert rule.shape == (S, S) and rule[0, 0] == 1.0 and rule[9, 3] == np.float32(1.0) / np.float32(10.0)
+  out, keep = oracle.corm_forward(q, k, v, rule)
+  assert keep.dtype == torch.bool and keep.shape == (1, 2, S)
+  assert torch.equal(out, oracle.attn_forward(q, k, v))
+  assert keep[..., 0].all()                                               # p_00 == 1 >= 1
+  # q == 0: every visible probability equals 1/(i+1) exactly, so every key is kept
+  _, keep0 = oracle.corm_forward(torch.zeros_like(q), k, v, rule)
+  assert keep0.all()
+  # an all-ones threshold keeps only keys that some row attends to with probability one: key 0 (row 0)
+  ones = torch.ones(S, S)
+  _, keep1 = oracle.corm_forward(q, k, v, ones)
+  assert keep1[..., 0].all() and not keep1[..., 1:].any()
+  # fp64 brute force wherever the decision is not within 1e-3 of the boundary
+  ratio = brute.corm_ratio(q, k, rule)
+  clear = np.abs(ratio - 1.0) > 1e-3
+  assert clear.mean() > 0.9
+  assert np.array_equal(keep.numpy()[clear], (ratio >= 1.0)[clear])
+  assert 0.05 < keep.float().mean().item() < 0.999                         # the test exercises both outcomes
+  m = oracle.corm_margin(q, k, rule)
+  np.testing.assert_allclose(m.numpy(), ratio, rtol=3e-3)
+  assert torch.equal(m >= 1, keep) or (np.abs(m.numpy() - 1) < 1e-6).any()
+
+
+def test_gemma2_softcap_limits_and_brute_force():
+  q, k, v = _inputs(S=48, H=2, D=64, seed=13)
+  # a large power-of-two cap: logit / cap is exact unless it falls into fp16 subnormals (|logit| < 0.03),
+  # tanh(y) == y in fp16 for |y| < 0.027, times cap is exact -> plain attention up to a few last-bit flips
+  big = oracle.gemma2_forward(q, k, v, softcap=512.0)
+  plain = oracle.attn_forward(q, k, v)
+  assert (big.float() - plain.float()).abs().max().item() <= 2e-3
+  assert (big == plain).float().mean().item() > 0.99
+  # a tiny cap squashes every logit to (-cap, cap): probabilities ~ uniform over the visible prefix
+  o_small = oracle.gemma2_forward(q, k, v, softcap=1e-3)
+  prefix = torch.cumsum(v.float(), dim=1) / torch.arange(1, 49).view(1, -1, 1, 1)
+  assert (o_small.float() - prefix).abs().max().item() < 5e-3
+  ref = brute.softcap_attention(q, k, v, 50.0)
+  assert np.abs(oracle.gemma2_forward(q, k, v).float().numpy() - ref).max() < 4e-3
+  # the cap matters: with cap 2 the result differs clearly from plain attention and matches the brute force
+  ref2 = brute.softcap_attention(q, k, v, 2.0)
+  o2 = oracle.gemma2_forward(q, k, v, softcap=2.0).float().numpy()
+  assert np.abs(o2 - ref2).max() < 4e-3
+  assert np.abs(o2 - oracle.attn_forward(q, k, v).float().numpy()).max() > 2e-2
