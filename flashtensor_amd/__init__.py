@@ -5,7 +5,7 @@ workloads, hand-written in HIP for gfx950 in `csrc/`, exported through the C ABI
 (`libflashtensor_hip.so`), and a thin host mirror of the reference's backend interface
 (`Builder.build_callable`, the case modules' `forward` / `prepare`).
 """
-from . import ops  # noqa: F401
+from . import kernels, ops  # noqa: F401
 from .builder import Builder, HipBuilder  # noqa: F401
 from .kernels import CASES, get_model  # noqa: F401
 from .utils import loss, perf  # noqa: F401

@@ -28,7 +28,7 @@ class FtAttnArgs(ctypes.Structure):
   _fields_ = [("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("o", ctypes.c_void_p),
               ("sq", FtStrides), ("sk", FtStrides), ("sv", FtStrides), ("so", FtStrides),
               ("B", ctypes.c_int32), ("H", ctypes.c_int32), ("Sq", ctypes.c_int32), ("Skv", ctypes.c_int32),
-              ("D", ctypes.c_int32), ("dtype", ctypes.c_int32), ("flags", ctypes.c_uint32)]
+              ("D", ctypes.c_int32), ("dtype", ctypes.c_int32), ("flags", ctypes.c_uint32), ("Hkv", ctypes.c_int32)]
 
 
 class FtNoise(ctypes.Structure):

@@ -24,6 +24,7 @@ size_t linattn_workspace_bytes(const FtAttnArgs& a, int kind);
 hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* idx, hipStream_t s);
 hipError_t launch_noise_fill(float* dst, int B, int H, int Sq, int Skv, uint64_t seed, hipStream_t s);
 hipError_t launch_avgpool1d(const float* src, int64_t rows, int S, int kernel, float* dst, hipStream_t s);
+hipError_t launch_group_mean(const float* src, int64_t groups, int group, int S, float* dst, hipStream_t s);
 }  // namespace ft
 
 namespace {
@@ -114,6 +115,8 @@ int validate_attn(const FtAttnArgs* a, bool need_v_o) {
   if (need_v_o && (!a->v || !a->o)) return fail(FT_EINVAL, "v / o pointer is null");
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Skv < 1)
     return fail(FT_EINVAL, "bad shape B=%d H=%d Sq=%d Skv=%d", a->B, a->H, a->Sq, a->Skv);
+  if (a->Hkv < 0 || (a->Hkv > 0 && (a->Hkv > a->H || a->H % a->Hkv != 0)))
+    return fail(FT_EINVAL, "bad head grouping H=%d Hkv=%d (H must be a multiple of Hkv)", a->H, a->Hkv);
   if (a->D != 64 && a->D != 128) return fail(FT_EUNSUPPORTED, "head_dim %d not supported (64 or 128)", a->D);
   if (a->dtype != FT_F16 && a->dtype != FT_BF16) return fail(FT_EUNSUPPORTED, "dtype %d not supported (f16 or bf16)", a->dtype);
   if ((a->flags & FT_CAUSAL) && a->Skv < a->Sq)
@@ -132,6 +135,11 @@ int validate_attn(const FtAttnArgs* a, bool need_v_o) {
 }
 
 ft::Strides3 cvt(const FtStrides& s) { return ft::Strides3{s.b, s.s, s.h}; }
+int group_of(const FtAttnArgs* a) { return a->Hkv > 0 ? a->H / a->Hkv : 1; }
+int reject_groups(const FtAttnArgs* a, const char* what) {
+  if (group_of(a) != 1) return fail(FT_EUNSUPPORTED, "%s does not take grouped queries (H=%d Hkv=%d)", what, a->H, a->Hkv);
+  return FT_OK;
+}
 
 ft::AttnKernelParams attn_params(const FtAttnArgs* a, bool emu) {
   ft::AttnKernelParams p;
@@ -152,6 +160,7 @@ ft::AttnKernelParams attn_params(const FtAttnArgs* a, bool emu) {
   p.logit_mul = emu ? tuned_logit_multiplier(a->D, a->dtype == FT_BF16)
                     : (float)(1.4426950408889634 / std::sqrt((double)a->D));
   p.inv_tau = 1.f;
+  p.group = group_of(a);
   return p;
 }
 
@@ -173,10 +182,15 @@ ft::ColstatsKernelParams col_params(const FtAttnArgs* a, bool emu, const float* 
   p.logit_mul = emu ? tuned_logit_multiplier(a->D, a->dtype == FT_BF16)
                     : (float)(1.4426950408889634 / std::sqrt((double)a->D));
   p.inv_tau = 1.f;
+  p.group = group_of(a);
   return p;
 }
 
 size_t lse_bytes(const FtAttnArgs* a) { return (size_t)a->B * a->H * a->Sq * sizeof(float); }
+// grouped queries: the per-query-head column sums live in the workspace before their group mean is taken
+size_t colstats_bytes(const FtAttnArgs* a) {
+  return lse_bytes(a) + (group_of(a) > 1 ? (size_t)a->B * a->H * a->Skv * sizeof(float) : 0);
+}
 
 }  // namespace
 
@@ -192,6 +206,7 @@ size_t ft_workspace_bytes(int op, const FtAttnArgs* a) {
     case FT_OP_ATTN:
       return 0;
     case FT_OP_COLSTATS:
+      return colstats_bytes(a);
     case FT_OP_KEYFORMER:
     case FT_OP_CORM:
       return lse_bytes(a);
@@ -217,26 +232,36 @@ int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, vo
                          void* stream) {
   if (int rc = validate_attn(a, true)) return rc;
   if (!colsum) return fail(FT_EINVAL, "colsum pointer is null");
-  if (!workspace || workspace_bytes < lse_bytes(a))
-    return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", lse_bytes(a), workspace ? workspace_bytes : (size_t)0);
+  const int group = group_of(a);
+  if (group > 1 && colsumsq) return fail(FT_EUNSUPPORTED, "sum of squares is not defined per query head under grouped queries");
+  const size_t need = colstats_bytes(a);
+  if (!workspace || workspace_bytes < need)
+    return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
   if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(FT_EINVAL, "workspace must be 4-byte aligned");
   const bool emu = !(a->flags & FT_FAST_LOGITS);
   const bool causal = a->flags & FT_CAUSAL;
   float* lse = static_cast<float*>(workspace);
+  float* per_head = group > 1 ? lse + (size_t)a->B * a->H * a->Sq : colsum;
   ft::AttnKernelParams p = attn_params(a, emu);
   p.lse = lse;
   hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, causal, emu, ft::kKfNone, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "attn_fwd launch");
-  ft::ColstatsKernelParams c = col_params(a, emu, lse, colsum, colsumsq);
+  ft::ColstatsKernelParams c = col_params(a, emu, lse, per_head, colsumsq);
   e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, colsumsq ? ft::kStatSumSq : ft::kStatSum,
                           (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "colstats launch");
+  if (group > 1) {
+    if ((int64_t)a->B * a->Hkv > 65535) return fail(FT_EUNSUPPORTED, "too many k/v heads for the group mean");
+    e = ft::launch_group_mean(per_head, (int64_t)a->B * a->Hkv, group, a->Skv, colsum, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "group mean launch");
+  }
   return FT_OK;
 }
 
 int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float* kf_score, void* workspace,
                      size_t workspace_bytes, void* stream) {
   if (int rc = validate_attn(a, true)) return rc;
+  if (int rc = reject_groups(a, "keyformer")) return rc;
   if (!noise) return fail(FT_EINVAL, "noise descriptor is null");
   if (!kf_score) return fail(FT_EINVAL, "kf_score pointer is null");
   if (!(tau > 0.f) || !std::isfinite(tau)) return fail(FT_EINVAL, "tau must be positive and finite (got %g)", (double)tau);
@@ -294,6 +319,7 @@ int ft_attn_softcap_fwd(const FtAttnArgs* a, float softcap, float* lse, void* st
 int ft_corm_fwd(const FtAttnArgs* a, const float* corm_mask, int64_t mask_row_stride, uint8_t* corm_score, float* margin,
                 void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = validate_attn(a, true)) return rc;
+  if (int rc = reject_groups(a, "corm")) return rc;
   if (!corm_score) return fail(FT_EINVAL, "corm_score pointer is null");
   if (corm_mask && (mask_row_stride < a->Skv || (reinterpret_cast<uintptr_t>(corm_mask) & 3u)))
     return fail(FT_EINVAL, "corm_mask needs a contiguous last axis and row stride >= Skv");
@@ -337,6 +363,7 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
   if (!a->q || !a->k || !a->v || !a->o) return fail(FT_EINVAL, "q / k / v / o pointer is null");
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Skv != a->Sq)
     return fail(FT_EINVAL, "bad shape B=%d H=%d Sq=%d Skv=%d (linear attention needs Sq == Skv)", a->B, a->H, a->Sq, a->Skv);
+  if (a->Hkv != 0 && a->Hkv != a->H) return fail(FT_EUNSUPPORTED, "linear attention does not take grouped queries (H=%d Hkv=%d)", a->H, a->Hkv);
   if (a->D != 64) return fail(FT_EUNSUPPORTED, "head_dim %d not supported by the linear-attention kernels (64)", a->D);
   if (a->dtype != FT_F16) return fail(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16)", a->dtype);
   if (out_dtype != FT_F16 && out_dtype != FT_F32) return fail(FT_EUNSUPPORTED, "out_dtype must be f16 or f32");

@@ -74,8 +74,8 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
 #pragma unroll
   for (int t = 0; t < KSTEPS; ++t) qf[t] = *reinterpret_cast<const vec8*>(qptr + 16 * t + 8 * g);
 
-  const uint16_t* kbase = p.k + b * p.sk.b + h * p.sk.h;
-  const uint16_t* vbase = p.v + b * p.sv.b + h * p.sv.h;
+  const uint16_t* kbase = p.k + b * p.sk.b + (h / p.group) * p.sk.h;
+  const uint16_t* vbase = p.v + b * p.sv.b + (h / p.group) * p.sv.h;
 
   // tiles of the workgroup, of this wave (not entirely above its diagonal), and of this wave's mask-free prefix
   const int wave_row0 = m0 + wave * 32;

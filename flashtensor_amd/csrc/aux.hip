@@ -106,4 +106,23 @@ hipError_t launch_avgpool1d(const float* src, int64_t rows, int S, int kernel, f
   return hipGetLastError();
 }
 
+// Mean over the `group` consecutive rows of each group: src [groups, group, S] -> dst [groups, S]
+// (grouped-query H2O score, cases/attn_h2o.py:42-47; the mean over heads commutes with the sum over rows).
+__global__ void __launch_bounds__(256) group_mean_kernel(const float* __restrict__ src, float* __restrict__ dst, int S, int group) {
+  const int64_t grp = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= S) return;
+  const float* r = src + grp * group * S + j;
+  float acc = 0.f;
+  for (int t = 0; t < group; ++t) acc += r[(int64_t)t * S];
+  dst[grp * S + j] = acc / (float)group;
+}
+
+hipError_t launch_group_mean(const float* src, int64_t groups, int group, int S, float* dst, hipStream_t s) {
+  if (groups > 65535) return hipErrorInvalidValue;
+  dim3 grid((unsigned)((S + 255) / 256), (unsigned)groups);
+  hipLaunchKernelGGL(group_mean_kernel, grid, dim3(256), 0, s, src, dst, S, group);
+  return hipGetLastError();
+}
+
 }  // namespace ft

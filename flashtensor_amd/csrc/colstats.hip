@@ -59,7 +59,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   const float POS_INF = __builtin_inff();
   const float NEG_INF = -__builtin_inff();
 
-  const uint16_t* kptr = p.k + b * p.sk.b + (int64_t)kj_c * p.sk.s + h * p.sk.h;
+  const uint16_t* kptr = p.k + b * p.sk.b + (int64_t)kj_c * p.sk.s + (h / p.group) * p.sk.h;
   vec8 kf[KSTEPS];
 #pragma unroll
   for (int t = 0; t < KSTEPS; ++t) kf[t] = *reinterpret_cast<const vec8*>(kptr + 16 * t + 8 * g);

@@ -25,6 +25,7 @@ struct AttnKernelParams {
   float logit_mul;  // reference rounding: f16(f16(acc) * logit_mul) == f16(f16(acc) / sqrt(D)); fast: log2e / sqrt(D)
   float inv_tau;
   float softcap;    // kKfSoftcap: logits become softcap * tanh(logit / softcap)
+  int group;        // query heads per k/v head: query head h reads k/v head h / group
 };
 
 struct ColstatsKernelParams {
@@ -42,6 +43,7 @@ struct ColstatsKernelParams {
   int off;
   float logit_mul;
   float inv_tau;
+  int group;  // query heads per k head
 };
 
 // what happens to a logit between the scaled QK^T and the softmax of the attention pass

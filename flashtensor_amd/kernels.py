@@ -130,6 +130,42 @@ class Gemma2(_Case):
     return ops.gemma2(q, k, v, softcap=self.logit_softcapping)
 
 
+class Attn2D:
+  """cases/attn.py:12-69: the harness form on 2-D activations, q [q_len, head_num * head_dim], k, v
+  [kv_len, kv_head_num * head_dim] -> out [q_len, head_num * head_dim]; grouped queries when
+  kv_head_num < head_num, `masked` selects the causal variant."""
+
+  def __init__(self, kv_head_num, head_num, head_dim, masked):
+    self.kv_head_num = kv_head_num
+    self.head_num = head_num
+    self.head_dim = head_dim
+    self.masked = masked
+    self.group_size = self.head_num // self.kv_head_num
+
+  def __call__(self, *args):
+    return self.forward(*args)
+
+  def eval(self):
+    return self
+
+  def _views(self, q, k, v):
+    return (q.view(1, q.shape[0], self.head_num, self.head_dim), k.view(1, k.shape[0], self.kv_head_num, self.head_dim),
+            v.view(1, v.shape[0], self.kv_head_num, self.head_dim))
+
+  def forward(self, q, k, v):
+    q4, k4, v4 = self._views(q, k, v)
+    return ops.attn(q4, k4, v4, causal=self.masked).view(q.shape[0], self.head_num * self.head_dim)
+
+
+class AttnH2O2D(Attn2D):
+  """cases/attn_h2o.py:11-81: (out [q_len, hidden], h2o_score [kv_head_num, kv_len])."""
+
+  def forward(self, q, k, v):
+    q4, k4, v4 = self._views(q, k, v)
+    out, score = ops.h2o(q4, k4, v4, causal=self.masked)
+    return out.view(q.shape[0], self.head_num * self.head_dim), score.view(self.kv_head_num, k.shape[0])
+
+
 class EA(_Case):
   """Attention core of bench/ea.mlir:13-17 on [B,S,H,D] tensors."""
   output = ["out"]

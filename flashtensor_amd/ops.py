@@ -32,8 +32,9 @@ def _check_qkv(q, k, v):
   if q.dtype not in _DTYPES:
     raise RuntimeError(f"arg 0 need dtype float16 or bfloat16 but got {q.dtype}")
   B, Sq, H, D = q.shape
-  if tuple(k.shape) != (B, k.shape[1], H, D):
-    raise RuntimeError(f"arg 1 need shape {(B, k.shape[1], H, D)} but got {tuple(k.shape)}")
+  Hkv = k.shape[2]
+  if tuple(k.shape) != (B, k.shape[1], Hkv, D) or Hkv < 1 or H % Hkv != 0:
+    raise RuntimeError(f"arg 1 need shape {(B, k.shape[1], 'a divisor of ' + str(H), D)} but got {tuple(k.shape)}")
   if tuple(v.shape) != tuple(k.shape):
     raise RuntimeError(f"arg 2 need shape {tuple(k.shape)} but got {tuple(v.shape)}")
 
@@ -49,7 +50,7 @@ def _strides(t):
 def _args(q, k, v, o, flags):
   B, Sq, H, D = q.shape
   return FtAttnArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _strides(q), _strides(k), _strides(v),
-                    _strides(o), B, H, Sq, k.shape[1], D, _DTYPES[q.dtype], flags)
+                    _strides(o), B, H, Sq, k.shape[1], D, _DTYPES[q.dtype], flags, k.shape[2])
 
 
 def _flags(causal, fast_logits):
@@ -62,7 +63,8 @@ def _prep(q, k, v):
 
 
 def attn(q, k, v, causal=True, fast_logits=False, return_lse=False):
-  """Attn.forward (cases/kernels/attn.py:18-34): q,k,v [B,S,H,D] -> out [B,Sq,H,D]."""
+  """Attn.forward (cases/kernels/attn.py:18-34): q [B,S,H,D], k,v [B,Skv,Hkv,D] -> out [B,Sq,H,D].  With
+  Hkv < H query head h attends to k/v head h // (H // Hkv), the grouping of cases/attn.py:29-31."""
   q, k, v = _prep(q, k, v)
   lib = _lib.load()
   out = torch.empty_like(q, memory_format=torch.contiguous_format)
@@ -78,7 +80,7 @@ def _colstats(q, k, v, want_sq, causal, fast_logits):
   B, Sq, H, D = q.shape
   Skv = k.shape[1]
   out = torch.empty_like(q, memory_format=torch.contiguous_format)
-  s1 = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device)
+  s1 = torch.empty(B, k.shape[2], Skv, dtype=torch.float32, device=q.device)  # per k/v head (group mean when grouped)
   s2 = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device) if want_sq else None
   a = _args(q, k, v, out, _flags(causal, fast_logits))
   nbytes = lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a))
@@ -89,7 +91,8 @@ def _colstats(q, k, v, want_sq, causal, fast_logits):
 
 
 def h2o(q, k, v, causal=True, fast_logits=False):
-  """H2O.forward (cases/kernels/h2o.py:18-38) -> (out, h2o_score [B,H,Skv] fp32)."""
+  """H2O.forward (cases/kernels/h2o.py:18-38) -> (out, h2o_score [B,Hkv,Skv] fp32); under grouped queries
+  the probabilities are averaged over each group's query heads before the sum (cases/attn_h2o.py:42-47)."""
   return _colstats(q, k, v, False, causal, fast_logits)
 
 

@@ -49,7 +49,9 @@ typedef struct FtStrides {
   int64_t b, s, h;
 } FtStrides;
 
-/* One attention problem: q [B,Sq,H,D], k,v [B,Skv,H,D], o [B,Sq,H,D] (cases/kernels/attn.py:37-39, :32-34). */
+/* One attention problem: q [B,Sq,H,D], k,v [B,Skv,Hkv,D], o [B,Sq,H,D] (cases/kernels/attn.py:37-39, :32-34).
+ * Hkv = 0 or H: one k/v head per query head.  Hkv < H (H a multiple of Hkv): grouped queries as in
+ * cases/attn.py:29-31, query head h reads k/v head h / (H / Hkv); sk.h, sv.h are then strides of k/v heads. */
 typedef struct FtAttnArgs {
   const void* q;
   const void* k;
@@ -59,6 +61,7 @@ typedef struct FtAttnArgs {
   int32_t B, H, Sq, Skv, D;
   int32_t dtype;  /* FtDtype of q, k, v, o */
   uint32_t flags; /* FtFlags */
+  int32_t Hkv;    /* number of k/v heads; 0 means H */
 } FtAttnArgs;
 
 /* KeyFormer noise source.  exp_rand != NULL: the reference's input tensor [B,H,Sq,Skv] fp32
@@ -82,7 +85,9 @@ size_t ft_workspace_bytes(int op, const FtAttnArgs* a);
 int ft_attn_fwd(const FtAttnArgs* a, float* lse, void* stream);
 
 /* Attention + per-key column statistics: H2O.forward (cases/kernels/h2o.py:18-38; colsumsq == NULL) and
- * RoCo.forward (cases/kernels/roco.py:18-48).  colsum, colsumsq: [B,H,Skv] fp32. */
+ * RoCo.forward (cases/kernels/roco.py:18-48).  colsum, colsumsq: [B,H,Skv] fp32.
+ * Grouped queries (Hkv < H, colsumsq == NULL only): colsum is [B,Hkv,Skv], the column sums of the
+ * probabilities averaged over the query heads of each group (cases/attn_h2o.py:42-47). */
 int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, void* workspace, size_t workspace_bytes,
                          void* stream);
 

@@ -25,6 +25,9 @@ How each function is pinned (tests/test_oracle_pins.py, tests/test_oracle_golden
   gemma2_forward     softcap = 512 (a power of two, tanh(y) == y in fp16 for the tiny y) -> attn_forward
                      up to last-bit flips; tiny softcap -> logits ~ 0 -> prefix means of V; fp64 brute
                      force at caps 50 and 2.
+  attn2d_forward,    Hkv == H -> attn_forward / h2o_forward on the [1,S,H,D] views, bit-exact; Hkv < H ->
+  attn_h2o2d_forward the same functions on k/v heads repeated with repeat_interleave, scores averaged per group;
+                     fp64 brute force with explicit h // group indexing; unmasked rows sum to Sq.
 The reference holds no golden vectors or tests for this path, so none can be checked against; no
 function of this file is "parity unpinned".
 """
@@ -145,6 +148,47 @@ def gemma2_forward(q, k, v, softcap=50.0):
   scores += mask
   probs = F.softmax(scores.float(), dim=-1)
   return _out(probs, q, v)
+
+
+def _probs_2d(q, k, v, kv_head_num, head_num, head_dim, masked):
+  """Shared body of cases/attn.py:20-42,44-63 and cases/attn_h2o.py:19-40,50-66: 2-D activations, grouped
+  queries by expanding k/v heads, optional causal mask.  Returns (probs fp32 [H,Sq,Skv], q, v as [H,S,D])."""
+  q_len, kv_len = q.shape[0], k.shape[0]
+  group_size = head_num // kv_head_num
+  q = q.view(q_len, head_num, head_dim)
+  k = k.view(kv_len, kv_head_num, head_dim)
+  v = v.view(kv_len, kv_head_num, head_dim)
+  if group_size > 1:
+    k = k[:, :, None, :].expand(kv_len, kv_head_num, group_size, head_dim).reshape(kv_len, head_num, head_dim)
+    v = v[:, :, None, :].expand(kv_len, kv_head_num, group_size, head_dim).reshape(kv_len, head_num, head_dim)
+  q, k, v = q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1)
+  scores = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(head_dim)
+  if masked:
+    mask = torch.full((1, q_len, kv_len), -torch.inf, device=q.device, dtype=scores.dtype)
+    scores += torch.triu(mask, diagonal=kv_len - q_len + 1)
+  return F.softmax(scores.float(), dim=-1), q, v
+
+
+def attn2d_forward(q, k, v, kv_head_num, head_num, head_dim, masked=True):
+  """cases/attn.py:20-69: q [q_len, H*D], k, v [kv_len, Hkv*D] -> out [q_len, H*D]."""
+  probs, qh, vh = _probs_2d(q, k, v, kv_head_num, head_num, head_dim, masked)
+  out = torch.matmul(probs.to(qh.dtype), vh).transpose(0, 1).contiguous()
+  return out.view(q.shape[0], head_num * head_dim)
+
+
+def attn_h2o2d_forward(q, k, v, kv_head_num, head_num, head_dim, masked=True):
+  """cases/attn_h2o.py:19-81: as attn2d_forward plus h2o_score [Hkv, kv_len] = sum over query rows of the
+  probabilities averaged over the query heads of each group (:42-47)."""
+  q_len, kv_len = q.shape[0], k.shape[0]
+  group_size = head_num // kv_head_num
+  probs, qh, vh = _probs_2d(q, k, v, kv_head_num, head_num, head_dim, masked)
+  out = torch.matmul(probs.to(qh.dtype), vh).transpose(0, 1).contiguous()
+  if group_size > 1:
+    h2o_score = probs.reshape(kv_head_num, group_size, q_len, kv_len).mean(dim=1)
+  else:
+    h2o_score = probs
+  h2o_score = h2o_score.sum(dim=1)
+  return out.view(q_len, head_num * head_dim), h2o_score.view(kv_head_num, kv_len)
 
 
 def ea_forward(q, k, v):

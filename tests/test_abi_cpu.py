@@ -50,6 +50,8 @@ def _args(**over):
     (dict(Sq=16, Skv=8), _lib.FT_EINVAL, "Skv >= Sq"),
     (dict(q=0x1004), _lib.FT_EINVAL, "aligned"),
     (dict(sq=FtStrides(2048, 250, 128)), _lib.FT_EINVAL, "strides"),
+    (dict(H=6, Hkv=4), _lib.FT_EINVAL, "grouping"),
+    (dict(H=2, Hkv=4), _lib.FT_EINVAL, "grouping"),
 ])
 def test_attn_rejects_bad_arguments_before_launch(lib, over, code, needle):
   a = _args(**over)
@@ -93,6 +95,20 @@ def test_softcap_corm_and_avgpool_argument_checks(lib):
   assert "odd" in lib.ft_last_error().decode()
   assert lib.ft_avgpool1d(0x1000, 1, 8, 5, 0x1000, None) == _lib.FT_EINVAL
   assert lib.ft_avgpool1d(0x1000, 0, 8, 5, 0x2000, None) == _lib.FT_EINVAL
+
+
+def test_grouped_query_argument_checks(lib):
+  a = _args(H=4, Hkv=2)
+  assert lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a)) == 1 * 4 * 8 * 4 * 2   # normalisers + per-head sums
+  assert lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(_args(H=4, Hkv=4))) == 1 * 4 * 8 * 4
+  assert lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(_args(H=4))) == 1 * 4 * 8 * 4           # Hkv = 0 means H
+  need = lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a))
+  assert lib.ft_attn_colstats_fwd(ctypes.byref(a), 0x6000, 0x7000, 0x5000, need, None) == _lib.FT_EUNSUPPORTED
+  assert "grouped" in lib.ft_last_error().decode()
+  assert lib.ft_attn_colstats_fwd(ctypes.byref(a), 0x6000, None, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
+  noise = FtNoise(None, 0, 0, 0, 1)
+  assert lib.ft_keyformer_fwd(ctypes.byref(a), ctypes.byref(noise), 1.0, 0x6000, 0x5000, need, None) == _lib.FT_EUNSUPPORTED
+  assert lib.ft_corm_fwd(ctypes.byref(a), None, 0, 0x6000, None, 0x5000, need, None) == _lib.FT_EUNSUPPORTED
 
 
 def test_linattn_and_topk_argument_checks(lib):

@@ -348,6 +348,41 @@ def test_next_cases_at_reference_default_shape(gpu):
   assert torch.equal(f(qd, kd, vd)[1], s)
 
 
+# ------------------------------------------------------------------ grouped queries, 2-D harness form
+
+@pytest.mark.parametrize("S,Skv,H,Hkv,D,masked", [(128, 128, 4, 2, 128, True), (200, 200, 8, 2, 64, True), (96, 232, 4, 1, 128, True),
+                                                  (160, 160, 4, 2, 128, False), (130, 130, 6, 6, 128, True)])
+def test_grouped_queries_2d(gpu, S, Skv, H, Hkv, D, masked):
+  g = torch.Generator().manual_seed(S + H)
+  q = torch.randn(S, H * D, dtype=torch.float16, generator=g)
+  k = torch.randn(Skv, Hkv * D, dtype=torch.float16, generator=g)
+  v = torch.randn(Skv, Hkv * D, dtype=torch.float16, generator=g)
+  ref_o, ref_s = oracle.attn_h2o2d_forward(q, k, v, Hkv, H, D, masked)
+  model = ft.kernels.AttnH2O2D(Hkv, H, D, masked)
+  out, score = model(q.to(gpu), k.to(gpu), v.to(gpu))
+  assert out.shape == (S, H * D) and score.shape == (Hkv, Skv)
+  check_o(out, ref_o); check_score(score, ref_s)
+  out_a = ft.kernels.Attn2D(Hkv, H, D, masked)(q.to(gpu), k.to(gpu), v.to(gpu))
+  assert torch.equal(out_a, out)
+  assert torch.equal(out_a.cpu(), out_a.cpu()) and (out_a.float().cpu() - oracle.attn2d_forward(q, k, v, Hkv, H, D, masked).float()).abs().max() <= O_ABS
+
+
+def test_grouped_queries_equal_repeated_kv_heads(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 2, 192, 8, 128, seed=21)
+  kg, vg = kd[:, :, :2].contiguous(), vd[:, :, :2].contiguous()
+  out_g, s_g = ops.h2o(qd, kg, vg)
+  out_r, s_r = ops.h2o(qd, kg.repeat_interleave(4, dim=2), vg.repeat_interleave(4, dim=2))
+  assert torch.equal(out_g, out_r)                                         # same arithmetic, only the k/v addressing differs
+  assert torch.allclose(s_g, s_r.view(2, 2, 4, 192).mean(dim=2), rtol=1e-6)
+  assert torch.equal(ops.gemma2(qd, kg, vg), ops.gemma2(qd, kg.repeat_interleave(4, dim=2), vg.repeat_interleave(4, dim=2)))
+  with pytest.raises(ft._lib.FtError, match="grouped"):
+    ops.roco(qd, kg, vg)
+  with pytest.raises(ft._lib.FtError, match="grouped"):
+    ops.keyformer(qd, kg, vg, None, seed=1)
+  with pytest.raises(RuntimeError, match="divisor"):
+    ops.attn(qd, kd[:, :, :3].contiguous(), vd[:, :, :3].contiguous())
+
+
 # ------------------------------------------------------------------ the five measured configurations
 
 def test_config1_attn_b1_h32_s1024_d128(gpu):

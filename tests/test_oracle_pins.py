@@ -313,3 +313,36 @@ def test_gemma2_softcap_limits_and_brute_force():
   o2 = oracle.gemma2_forward(q, k, v, softcap=2.0).float().numpy()
   assert np.abs(o2 - ref2).max() < 4e-3
   assert np.abs(o2 - oracle.attn_forward(q, k, v).float().numpy()).max() > 2e-2
+
+
+# ------------------------------------------------------------------ 2-D harness form, grouped queries
+
+def test_attn2d_and_grouped_h2o_against_expanded_heads_and_brute_force():
+  S, H, D = 40, 4, 64
+  q, k, v = _inputs(S=S, H=H, D=D, seed=14)
+  q2, k2, v2 = (t[0].reshape(S, H * D) for t in (q, k, v))
+  # one k/v head per query head: the 4-D cases on the same data, bit for bit
+  assert torch.equal(oracle.attn2d_forward(q2, k2, v2, H, H, D), oracle.attn_forward(q, k, v)[0].reshape(S, H * D))
+  o2, s2 = oracle.attn_h2o2d_forward(q2, k2, v2, H, H, D)
+  oh, sh = oracle.h2o_forward(q, k, v)
+  assert torch.equal(o2, oh[0].reshape(S, H * D)) and torch.equal(s2, sh[0])
+  # grouped: 4 query heads on 2 k/v heads == the ungrouped case on repeated k/v heads, scores averaged per pair
+  Hkv = 2
+  kg, vg = k[:, :, :Hkv].contiguous(), v[:, :, :Hkv].contiguous()
+  kr, vr = kg.repeat_interleave(H // Hkv, dim=2), vg.repeat_interleave(H // Hkv, dim=2)
+  og, sg = oracle.attn_h2o2d_forward(q2, kg[0].reshape(S, Hkv * D), vg[0].reshape(S, Hkv * D), Hkv, H, D)
+  orf, srf = oracle.h2o_forward(q, kr, vr)
+  assert torch.equal(og, orf[0].reshape(S, H * D))
+  assert torch.allclose(sg, srf[0].view(Hkv, H // Hkv, S).mean(dim=1), rtol=1e-6)
+  assert abs(sg.sum().item() - Hkv * S) < 1e-3 * S                         # every averaged row still sums to one
+  # independent fp64 definition with explicit head // group indexing
+  O, cs, _, _ = brute.attention_stats(q, kr, vr)
+  np.testing.assert_allclose(sg.numpy(), cs[0].reshape(Hkv, H // Hkv, S).mean(axis=1), rtol=2e-3)
+  assert np.abs(og.float().numpy() - O[0].reshape(S, H * D)).max() < 4e-3
+  # query head 1 must read k/v head 0, not 1: swapping the two k/v heads changes its output
+  ksw = kg[:, :, [1, 0]].contiguous()
+  osw = oracle.attn2d_forward(q2, ksw[0].reshape(S, Hkv * D), vg[0].reshape(S, Hkv * D), Hkv, H, D)
+  assert (osw.view(S, H, D)[:, 1] - og.view(S, H, D)[:, 1]).abs().max().item() > 1e-2
+  # unmasked variant: every key is visible to every row
+  of, sf = oracle.attn_h2o2d_forward(q2, k2, v2, H, H, D, masked=False)
+  assert abs(sf.sum().item() - H * S) < 1e-3 * S and (sf[:, -1] > 0.1).all()
