@@ -73,6 +73,14 @@ def per_config_table(dev):
                lambda q, k, v: (lambda: ops.keyformer(q, k, v, er, tau=1.5)), extra_bytes=2 * er.numel() * 4)
   del er
   softmax_case("4 roco", 4, 4096, 32, 128, lambda q, k, v: (lambda: ops.roco(q, k, v)), extra_bytes=2 * 4 * 32 * 4096 * 4)
+  # the other cases of the reference's zoo at their prepare() defaults (B=1 H=32 S=4096 D=128)
+  softmax_case("snapkv k=5", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.snapkv(q, k, v)), extra_bytes=32 * 4096 * 4)
+  softmax_case("corm 1/(i+1)", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.corm(q, k, v)), extra_bytes=32 * 4096)
+  softmax_case("gemma2 cap=50", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.gemma2(q, k, v)))
+  q, k, v = qkv(1, 4096, 32, 128)
+  kg, vg = k[:, :, :8].contiguous(), v[:, :, :8].contiguous()
+  add("h2o grouped H32/Hkv8", "B1 H32 S4096 D128", lambda: ops.h2o(q, kg, vg), 2.0 * 32 * 4096 * 4096 * 128,
+      (2 * q.numel() + 2 * kg.numel()) * 2.0 + 8 * 4096 * 4)
   q, k, v = qkv(8, 8192, 16, 64)
   lin_flops, lin_bytes = 2 * 2.0 * 8 * 16 * 8192 * 64 * 64, 4.0 * 8 * 16 * 8192 * 64 * 2
   add("5 ea", "B8 H16 S8192 D64", lambda: ops.ea(q, k, v), lin_flops, lin_bytes)

@@ -21,6 +21,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # (name, B, S, H, D, seed)
 SHAPES = [("s128_d128", 1, 128, 2, 128, 0), ("s256_d64", 1, 256, 2, 64, 0), ("s200_d128", 1, 200, 2, 128, 1)]
 LIN_SHAPES = [("s256_d64", 1, 256, 2, 64, 0), ("s200_d64", 2, 200, 2, 64, 1)]
+NEXT_SHAPES = [("s128_d128", 1, 128, 2, 128, 3), ("s200_d64", 1, 200, 4, 64, 4)]
 KF_SEED = 1234
 
 
@@ -41,6 +42,19 @@ def main():
                         ea=oracle.ea_forward(q, k, v).numpy(),
                         sima=oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy(),
                         sima_rawq=oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32).numpy())
+  for name, B, S, H, D, seed in NEXT_SHAPES:
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+    rule = oracle.corm_mask_rule(S, S)
+    kg, vg = k[:, :, : H // 2].contiguous(), v[:, :, : H // 2].contiguous()  # grouped queries: two query heads per k/v head
+    og, sg = oracle.attn_h2o2d_forward(q[0].reshape(S, H * D), kg[0].reshape(S, H // 2 * D), vg[0].reshape(S, H // 2 * D),
+                                       H // 2, H, D)
+    np.savez_compressed(os.path.join(HERE, f"next_{name}.npz"), B=B, S=S, H=H, D=D, seed=seed,
+                        snapkv5=oracle.snapkv_forward(q, k, v)[1].numpy(),
+                        corm_keep=oracle.corm_forward(q, k, v, rule)[1].numpy(),
+                        corm_ratio=oracle.corm_margin(q, k, rule).numpy(),
+                        gemma2_cap50=oracle.gemma2_forward(q, k, v).numpy(),
+                        gemma2_cap2=oracle.gemma2_forward(q, k, v, softcap=2.0).numpy(),
+                        gqa_out=og.numpy(), gqa_score=sg.numpy())
   print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
 
 

@@ -177,6 +177,19 @@ def check_sima(out, ref, rel=1e-3):
   assert (out - ref).abs().max().item() <= rel * scale, f"sima {(out - ref).abs().max().item() / scale}"
 
 
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "next_*.npz"))), ids=os.path.basename)
+def test_next_cases_golden(gpu, path):
+  g = np.load(path, allow_pickle=False)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  _, (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  check_score(ops.snapkv(qd, kd, vd)[1], torch.from_numpy(g["snapkv5"]))
+  check_corm(ops.corm(qd, kd, vd)[1], torch.from_numpy(g["corm_ratio"]))
+  check_o(ops.gemma2(qd, kd, vd), torch.from_numpy(g["gemma2_cap50"]))
+  check_o(ops.gemma2(qd, kd, vd, softcap=2.0), torch.from_numpy(g["gemma2_cap2"]))
+  out, score = ops.h2o(qd, kd[:, :, : H // 2].contiguous(), vd[:, :, : H // 2].contiguous())
+  check_o(out[0].reshape(S, H * D), torch.from_numpy(g["gqa_out"])); check_score(score[0], torch.from_numpy(g["gqa_score"]))
+
+
 # ------------------------------------------------------------------ top-k heavy hitters
 
 def test_topk_matches_torch_and_orders_ties(gpu):

@@ -44,5 +44,24 @@ def test_linear_cases_match_golden(path):
                              g["sima_rawq"], rtol=1e-4, atol=1e-7)
 
 
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "next_*.npz"))), ids=os.path.basename)
+def test_next_cases_match_golden(path):
+  g = _load(path)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+  rule = oracle.corm_mask_rule(S, S)
+  np.testing.assert_allclose(oracle.snapkv_forward(q, k, v)[1].numpy(), g["snapkv5"], rtol=1e-5, atol=1e-7)
+  ratio = oracle.corm_margin(q, k, rule).numpy()
+  np.testing.assert_allclose(ratio, g["corm_ratio"], rtol=1e-5)
+  clear = np.abs(g["corm_ratio"] - 1) > 1e-4
+  assert np.array_equal(oracle.corm_forward(q, k, v, rule)[1].numpy()[clear], g["corm_keep"][clear])
+  assert np.abs(oracle.gemma2_forward(q, k, v).float().numpy() - g["gemma2_cap50"].astype(np.float32)).max() <= 2e-3
+  assert np.abs(oracle.gemma2_forward(q, k, v, softcap=2.0).float().numpy() - g["gemma2_cap2"].astype(np.float32)).max() <= 2e-3
+  kg, vg = k[:, :, : H // 2].contiguous(), v[:, :, : H // 2].contiguous()
+  og, sg = oracle.attn_h2o2d_forward(q[0].reshape(S, H * D), kg[0].reshape(S, H // 2 * D), vg[0].reshape(S, H // 2 * D), H // 2, H, D)
+  assert np.abs(og.float().numpy() - g["gqa_out"].astype(np.float32)).max() <= 2e-3
+  np.testing.assert_allclose(sg.numpy(), g["gqa_score"], rtol=1e-5, atol=1e-7)
+
+
 def test_golden_files_present():
-  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 5
+  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 7
