@@ -106,6 +106,33 @@ float tuned_logit_multiplier(int D, bool bf16) {
   return best;
 }
 
+// Packed-fp16 form of the division by sqrt(128) used by the fp16 fast paths: with hi = 0.70751953125 and
+// lo = -0.0004127025604248047 (both fp16), fma16(h, hi, mul16(h, lo)) == 8 * f16(h / sqrt(128)) for every finite
+// fp16 h whose quotient is at least 2.5e-3 in magnitude, and is within 2e-6 * 8 of it below (checked here over
+// all 65536 inputs on first use; a logit that small moves a probability by 2e-6 relative).  D = 64 needs no
+// constants: h / 8 is exact.
+bool packed_logit_constants(uint32_t* hi2, uint32_t* lo2) {
+  static int verified = 0;  // 0 unknown, 1 good, -1 bad
+  const _Float16 hi = (_Float16)0.70751953125f, lo = (_Float16)-0.0004127025604248047f;
+  if (verified == 0) {
+    bool ok = true;
+    const float c = (float)std::sqrt(128.0);
+    for (uint32_t bits = 0; bits < 65536 && ok; ++bits) {
+      const float x = half_bits_to_float((uint16_t)bits);
+      if (!std::isfinite(x)) continue;
+      const double want = (double)(float)(_Float16)(x / c);
+      const double cterm = (double)(float)(_Float16)((double)x * (double)(float)lo);
+      const double got = (double)(float)(_Float16)((double)x * (double)(float)hi + cterm) / 8.0;
+      if (got != want && (std::fabs(want) >= 2.5e-3 || std::fabs(got - want) > 2e-6)) ok = false;
+    }
+    verified = ok ? 1 : -1;
+  }
+  const uint16_t hb = float_to_half_bits((float)hi), lb = float_to_half_bits((float)lo);
+  *hi2 = (uint32_t)hb | ((uint32_t)hb << 16);
+  *lo2 = (uint32_t)lb | ((uint32_t)lb << 16);
+  return verified == 1;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 bool stride_ok(const FtStrides& s) { return s.b % 8 == 0 && s.s % 8 == 0 && s.h % 8 == 0 && s.s > 0; }
 
@@ -118,6 +145,10 @@ int validate_attn(const FtAttnArgs* a, bool need_v_o) {
   if (a->Hkv < 0 || (a->Hkv > 0 && (a->Hkv > a->H || a->H % a->Hkv != 0)))
     return fail(FT_EINVAL, "bad head grouping H=%d Hkv=%d (H must be a multiple of Hkv)", a->H, a->Hkv);
   if (a->D != 64 && a->D != 128) return fail(FT_EUNSUPPORTED, "head_dim %d not supported (64 or 128)", a->D);
+  {
+    uint32_t hi2, lo2;
+    if (!packed_logit_constants(&hi2, &lo2)) return fail(FT_EUNSUPPORTED, "internal: packed logit constants failed their exhaustive check");
+  }
   if (a->dtype != FT_F16 && a->dtype != FT_BF16) return fail(FT_EUNSUPPORTED, "dtype %d not supported (f16 or bf16)", a->dtype);
   if ((a->flags & FT_CAUSAL) && a->Skv < a->Sq)
     return fail(FT_EINVAL, "causal mask needs Skv >= Sq (got Sq=%d Skv=%d): rows without a visible key are undefined", a->Sq, a->Skv);
@@ -161,6 +192,7 @@ ft::AttnKernelParams attn_params(const FtAttnArgs* a, bool emu) {
                     : (float)(1.4426950408889634 / std::sqrt((double)a->D));
   p.inv_tau = 1.f;
   p.group = group_of(a);
+  packed_logit_constants(&p.pk_hi2, &p.pk_lo2);
   return p;
 }
 
@@ -183,6 +215,7 @@ ft::ColstatsKernelParams col_params(const FtAttnArgs* a, bool emu, const float* 
                     : (float)(1.4426950408889634 / std::sqrt((double)a->D));
   p.inv_tau = 1.f;
   p.group = group_of(a);
+  packed_logit_constants(&p.pk_hi2, &p.pk_lo2);
   return p;
 }
 

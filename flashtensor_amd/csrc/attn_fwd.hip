@@ -220,6 +220,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     constexpr bool MASKED = decltype(masked_tag)::value;
     const float neg_m = -m_run;
     const half2v ones = {(_Float16)1.f, (_Float16)1.f};
+    const half2v pk_hi = __builtin_bit_cast(half2v, p.pk_hi2), pk_lo = __builtin_bit_cast(half2v, p.pk_lo2);
     // local key index of register r is 32 mbk + 8 (r / 4) + 4 g + r % 4; it is visible iff <= lim + 4 g
     const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0 - 4 * g;
     uint4v pw[4];
@@ -228,19 +229,18 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
 #pragma unroll
     for (int blk = 0; blk < 4; ++blk) {
       const int mbk = blk >> 1, rb = (blk & 1) * 8;
-      half2v h2[4];
-      _Float16 t[8];
+      half2v t2[4];
       float x[8];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float2v a2 = {s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]};
-        h2[i] = __builtin_convertvector(a2, half2v);  // QK^T is an fp16 tensor in the reference
+        const half2v h2 = __builtin_convertvector(a2, half2v);  // QK^T is an fp16 tensor in the reference
+        // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
+        t2[i] = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) t[i] = (_Float16)((float)h2[i >> 1][i & 1] * p.logit_mul);  // ... divided by sqrt(D) in fp16
-#pragma unroll
       for (int i = 0; i < 8; ++i) {
-        x[i] = __builtin_fmaf((float)t[i], kLog2e, neg_m);
+        x[i] = __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m);
         if (MASKED) {
           const int jl = 32 * mbk + 8 * ((rb + i) >> 2) + ((rb + i) & 3);
           x[i] = (jl > lim) ? NEG_INF : x[i];

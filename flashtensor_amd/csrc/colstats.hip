@@ -154,6 +154,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
           er[mbk][r] = (i < p.Sq) ? er_col[(int64_t)i * p.er_sr] : 1.f;
         }
     }
+    const half2v pk_hi = __builtin_bit_cast(half2v, p.pk_hi2), pk_lo = __builtin_bit_cast(half2v, p.pk_lo2);
     // key kj is hidden from row i0 + il when kj > i0 + il + off, i.e. il < lim
     const int lim = kj - i0 - p.off - 4 * g;
 #pragma unroll
@@ -170,10 +171,10 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
           for (int e = 0; e < 4; e += 2) {
             const float2v a2 = {s[mbk][4 * q4 + e], s[mbk][4 * q4 + e + 1]};
             const half2v h2 = __builtin_convertvector(a2, half2v);         // QK^T is an fp16 tensor in the reference
-            const _Float16 t0 = (_Float16)((float)h2[0] * p.logit_mul);    // ... divided by sqrt(D) in fp16
-            const _Float16 t1 = (_Float16)((float)h2[1] * p.logit_mul);
-            x[e] = __builtin_fmaf((float)t0, kLog2e, nlse4[e]);
-            x[e + 1] = __builtin_fmaf((float)t1, kLog2e, nlse4[e + 1]);
+            // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
+            const half2v t2 = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
+            x[e] = __builtin_fmaf((float)t2[0], kLog2e / 8.f, nlse4[e]);
+            x[e + 1] = __builtin_fmaf((float)t2[1], kLog2e / 8.f, nlse4[e + 1]);
           }
         } else {
 #pragma unroll

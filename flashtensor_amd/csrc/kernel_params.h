@@ -24,6 +24,10 @@ struct AttnKernelParams {
   int off;          // Skv - Sq: query i sees keys j <= i + off when causal
   float logit_mul;  // reference rounding: f16(f16(acc) * logit_mul) == f16(f16(acc) / sqrt(D)); fast: log2e / sqrt(D)
   float inv_tau;
+  // packed fp16 form of the same division for D = 128 (two packed ops on element pairs instead of one
+  // mixed-precision multiply per element): t8 = fma(h, pk_hi, h * pk_lo) is 8 * f16(h / sqrt(D)) for every
+  // fp16 h except where |h / sqrt(D)| < 2.5e-3, and there within 2e-6 of it; both halves hold the constant
+  uint32_t pk_hi2, pk_lo2;
   float softcap;    // kKfSoftcap: logits become softcap * tanh(logit / softcap)
   int group;        // query heads per k/v head: query head h reads k/v head h / group
 };
@@ -42,6 +46,7 @@ struct ColstatsKernelParams {
   int B, H, Sq, Skv;
   int off;
   float logit_mul;
+  uint32_t pk_hi2, pk_lo2;  // as in AttnKernelParams
   float inv_tau;
   int group;  // query heads per k head
 };
