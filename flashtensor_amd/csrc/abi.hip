@@ -319,8 +319,19 @@ int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float
     p.er_sr = noise->stride_row;
     p.er_vec4 = aligned16(noise->exp_rand) && noise->stride_b % 4 == 0 && noise->stride_h % 4 == 0 && noise->stride_row % 4 == 0;
   }
-  hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, causal, emu, tensor ? ft::kKfTensor : ft::kKfSeeded,
-                                     (hipStream_t)stream);
+  // seeded noise, fp16, reference rounding: the packed path (tau == 1 needs 1 / E only; tau >= 0.25 keeps
+  // the perturbed sum inside fp32 range under the plain softmax's stabiliser); otherwise the generic path
+  int amode = tensor ? ft::kKfTensor : ft::kKfSeeded, cmode = tensor ? ft::kStatKfTensor : ft::kStatKfSeeded;
+  if (!tensor && emu && a->dtype == FT_F16) {
+    if (tau == 1.f) {
+      amode = ft::kKfSeededTau1;
+      cmode = ft::kStatKfSeededTau1;
+    } else if (tau >= 0.25f) {
+      amode = ft::kKfSeededFast;
+      cmode = ft::kStatKfSeededFast;
+    }
+  }
+  hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, causal, emu, amode, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "attn_fwd (keyformer) launch");
   ft::ColstatsKernelParams c = col_params(a, emu, lse_kf, kf_score, nullptr);
   c.inv_tau = 1.f / tau;
@@ -331,8 +342,7 @@ int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float
     c.er_sh = noise->stride_h;
     c.er_sr = noise->stride_row;
   }
-  e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, tensor ? ft::kStatKfTensor : ft::kStatKfSeeded,
-                          (hipStream_t)stream);
+  e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, cmode, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "colstats (keyformer) launch");
   return FT_OK;
 }

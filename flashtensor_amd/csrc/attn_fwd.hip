@@ -40,7 +40,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   typedef typename T::vec8 vec8;
   constexpr int TILE_BYTES = BN * G::RB;
   constexpr bool kIsF16 = __is_same(typename T::elem, _Float16);
-  constexpr bool kFastMasked = kIsF16 && EMU && KF == kKfNone;  // variants served by the packed-fp16 softmax
+  constexpr bool kKfFast = KF == kKfSeededTau1 || KF == kKfSeededFast;           // seeded noise inside the packed path
+  constexpr bool kSeeded = KF == kKfSeeded || kKfFast;
+  constexpr bool kFastMasked = kIsF16 && EMU && (KF == kKfNone || kKfFast);  // variants served by the packed-fp16 softmax
+  static_assert(!kKfFast || (kIsF16 && EMU), "the packed KeyFormer modes exist for fp16 with reference rounding only");
   // Software pipeline across tiles: the QK^T MFMAs of tile it+1 are issued in the same iteration as the
   // softmax (VALU) and PV MFMAs of tile it, so the matrix and vector pipes overlap inside one wave.
   // K therefore runs one tile ahead of V in LDS.
@@ -50,7 +53,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   __shared__ __align__(16) char ldsK1[TILE_BYTES];
   __shared__ __align__(16) char ldsV0[TILE_BYTES];
   __shared__ __align__(16) char ldsV1[TILE_BYTES];
-  __shared__ uint32_t ldsCol[2 * BN];  // noise column terms of the current / next tile
+  __shared__ __align__(16) uint32_t ldsCol[2 * BN];  // noise column terms of the current / next tile
 
   const int BH = p.B * p.H;
   const int nMB = (p.Sq + BM - 1) / BM;
@@ -87,13 +90,13 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     nw = min(ntiles, (wave_row0 + 31 + p.off) / BN + 1);
     n_fast = min(n_fast, (wave_row0 + p.off + 1) / BN);  // tiles with n0 + BN - 1 <= wave_row0 + off
   }
-  if (KF != kKfNone || !(kIsF16 && EMU)) n_fast = 0;  // only the fp16 reference-rounding path has a mask-free instance
+  if (!kFastMasked) n_fast = 0;  // only the packed fp16 path has a mask-free instance
   n_fast = min(n_fast, nw);
 
   NoiseKeys nk = {0, 0};
   uint32_t a_i = 0;
   const float* er_row = nullptr;
-  if (KF == kKfSeeded) {
+  if (kSeeded) {
     nk = noise_keys(p.seed, (uint32_t)bh);
     a_i = noise_row(nk, (uint32_t)qi);
   }
@@ -108,7 +111,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   };
   auto stage_v = [&](int t, char* dst) {
     if (t < ntiles) stV.issue(t * BN, min(BN, p.Skv - t * BN), dst);
-    if (KF == kKfSeeded && t < ntiles && threadIdx.x < BN)
+    if (kSeeded && t < ntiles && threadIdx.x < BN)
       ldsCol[(t & 1) * BN + threadIdx.x] = noise_col(nk, (uint32_t)(t * BN + threadIdx.x));
   };
 
@@ -178,6 +181,8 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     if (__any(grow)) {
       const float m_new = grow ? rowmax : m_run;
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      if (KF == kKfSeededTau1) l_kf *= alpha;
+      if (KF == kKfSeededFast) l_kf *= __builtin_amdgcn_exp2f((m_run - m_new) * p.inv_tau);
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
   };
   // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.
-  auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0) {
+  auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0, int buf) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const float neg_m = -m_run;
     const half2v ones = {(_Float16)1.f, (_Float16)1.f};
@@ -246,8 +251,27 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
           x[i] = (jl > lim) ? NEG_INF : x[i];
         }
       }
+      // KeyFormer, seeded: E = -ln u of the 8 (query, key) pairs; the column terms of keys
+      // 32 mbk + 8 (rb / 4 [+ 1]) + 4 g + [0..3] are two aligned groups of four in LDS
+      float ee[8];
+      if constexpr (kKfFast) {
+        const uint32_t* col = ldsCol + buf * BN + 32 * mbk + 2 * rb + 4 * g;
+        const uint4v c0 = *reinterpret_cast<const uint4v*>(col), c1 = *reinterpret_cast<const uint4v*>(col + 8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          ee[i] = -kLn2 * __builtin_amdgcn_logf(noise_uniform(a_i, i < 4 ? c0[i] : c1[i - 4]));
+        if constexpr (KF == kKfSeededFast) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)  // exp2(((t - m) log2e - log2 E) / tau); hidden keys carry x = -inf
+            l_kf += __builtin_amdgcn_exp2f((x[i] - __builtin_amdgcn_logf(ee[i])) * p.inv_tau);
+        }
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) x[i] = __builtin_amdgcn_exp2f(x[i]);
+      if constexpr (KF == kKfSeededTau1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) l_kf = __builtin_fmaf(x[i], __builtin_amdgcn_rcpf(ee[i]), l_kf);  // exp(t - m) / E
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float2v p2 = {x[2 * i], x[2 * i + 1]};
@@ -379,6 +403,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   auto fast_tile = [&](auto masked_tag, auto stage_tag, float16v (&s_cur)[2], float16v (&s_next)[2], const char* tk_next,
                        const char* tv, int n0, int it, char* k_dst, char* v_dst) {
     constexpr bool STAGE = decltype(stage_tag)::value;
+    constexpr int kValuGroup = kKfFast ? 16 : 6;  // vector instructions placed after each MFMA
     vec8 pb[4];
     // STAGE: the direct-to-LDS loads of K[it+2] and V[it+1] (both full tiles) are issued from inside this
     // block, one every few MFMAs.  Issued back to back they fill the texture-address queue (one 1 KB load
@@ -390,21 +415,23 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       stV.issue_full((it + 1) * BN, v_dst);
     }
     qk_part(s_next, tk_next, std::integral_constant<int, KSTEPS / 2>{}, std::integral_constant<int, KSTEPS>{});
-    fast_exp(masked_tag, s_cur, pb, n0);
+    if (kKfFast && STAGE && threadIdx.x < BN)  // column terms of tile it + 1 (the other half of ldsCol)
+      ldsCol[((it + 1) & 1) * BN + threadIdx.x] = noise_col(nk, (uint32_t)((it + 1) * BN + threadIdx.x));
+    fast_exp(masked_tag, s_cur, pb, n0, it & 1);
     pv(pb, tv);
     __builtin_amdgcn_sched_group_barrier(0x100, 6, 2);
 #pragma unroll
     for (int i = 0; i < KSTEPS; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
-      __builtin_amdgcn_sched_group_barrier(0x002, 6, 2);
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuGroup, 2);
     }
 #pragma unroll
     for (int i = 0; i < 4 * DB; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
       if (STAGE && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 2);
-      __builtin_amdgcn_sched_group_barrier(0x002, 6, 2);
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuGroup, 2);
     }
   };
 
@@ -498,9 +525,11 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       }
     if (g == 0 && p.lse) p.lse[(int64_t)bh * p.Sq + qi] = m_run + __builtin_amdgcn_logf(l_run);
   }
-  if (KF == kKfTensor || KF == kKfSeeded) {
+  if (KF == kKfTensor || kSeeded) {
     l_kf += xchg32(l_kf);
-    if (qi < p.Sq && g == 0) p.lse_kf[(int64_t)bh * p.Sq + qi] = m_kf + __builtin_amdgcn_logf(l_kf);
+    // packed modes: the perturbed sum shares the plain softmax's stabiliser, scaled by 1 / tau
+    const float base = KF == kKfSeededTau1 ? m_run : KF == kKfSeededFast ? m_run * p.inv_tau : m_kf;
+    if (qi < p.Sq && g == 0) p.lse_kf[(int64_t)bh * p.Sq + qi] = base + __builtin_amdgcn_logf(l_kf);
   }
 }
 
@@ -523,6 +552,12 @@ static hipError_t launch_td(const AttnKernelParams& p, bool causal, bool emu, in
   FT_CASE(true, true, kKfTensor) FT_CASE(true, false, kKfTensor) FT_CASE(false, true, kKfTensor) FT_CASE(false, false, kKfTensor)
   FT_CASE(true, true, kKfSeeded) FT_CASE(true, false, kKfSeeded) FT_CASE(false, true, kKfSeeded) FT_CASE(false, false, kKfSeeded)
   FT_CASE(true, true, kKfSoftcap) FT_CASE(true, false, kKfSoftcap) FT_CASE(false, true, kKfSoftcap) FT_CASE(false, false, kKfSoftcap)
+  if constexpr (std::is_same<T, F16>::value) {  // packed KeyFormer modes: fp16 with reference rounding only
+    if (emu) {
+      FT_CASE(true, true, kKfSeededTau1) FT_CASE(false, true, kKfSeededTau1)
+      FT_CASE(true, true, kKfSeededFast) FT_CASE(false, true, kKfSeededFast)
+    }
+  }
 #undef FT_CASE
   return hipErrorInvalidValue;
 }

@@ -38,7 +38,9 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   typedef TileGeom<D> G;
   typedef typename T::vec8 vec8;
   constexpr int TILE_BYTES = BQ * G::RB;
-  constexpr bool KFM = (MODE == kStatKfTensor || MODE == kStatKfSeeded);
+  constexpr bool KFM = (MODE == kStatKfTensor || MODE == kStatKfSeeded);                 // generic KeyFormer modes
+  constexpr bool KFP = (MODE == kStatKfSeededTau1 || MODE == kStatKfSeededFast);         // seeded noise in the packed path
+  constexpr bool kSeeded = MODE == kStatKfSeeded || KFP;
   constexpr bool CORM = (MODE == kStatCormRule || MODE == kStatCormTensor);
   constexpr bool kPacked = __is_same(typename T::elem, _Float16) && EMU;  // packed-fp16 rounding chain
   // one LDS object per buffer: reads of one do not wait for the direct-to-LDS loads in flight into the other
@@ -79,7 +81,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   NoiseKeys nk = {0, 0};
   uint32_t b_j = 0;
   const float* er_col = nullptr;
-  if (MODE == kStatKfSeeded) {
+  if (kSeeded) {
     nk = noise_keys(p.seed, (uint32_t)bh);
     b_j = noise_col(nk, (uint32_t)kj);
   }
@@ -110,7 +112,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
       // CoRM rule: p_ij >= 1 / (i + 1)  <=>  log2 p_ij + log2(i + 1) >= 0, so no exponential is needed
       if (MODE == kStatCormRule) nl += __builtin_amdgcn_logf((float)(i + 1));
       ldsLse[(t & 1) * BQ + threadIdx.x] = nl;
-      if (MODE == kStatKfSeeded) ldsRow[(t & 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)i);
+      if (kSeeded) ldsRow[(t & 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)i);
     }
   };
 
@@ -164,7 +166,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
         const int il0 = 32 * mbk + 8 * q4;  // + 4 g + e
         const float4v nlse4 = *reinterpret_cast<const float4v*>(ldsLse + buf * BQ + il0 + 4 * g);
         uint4v row4 = {0, 0, 0, 0};
-        if (MODE == kStatKfSeeded) row4 = *reinterpret_cast<const uint4v*>(ldsRow + buf * BQ + il0 + 4 * g);
+        if (kSeeded) row4 = *reinterpret_cast<const uint4v*>(ldsRow + buf * BQ + il0 + 4 * g);
         float x[4];
         if (kPacked && !KFM) {
 #pragma unroll
@@ -173,8 +175,16 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
             const half2v h2 = __builtin_convertvector(a2, half2v);         // QK^T is an fp16 tensor in the reference
             // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
             const half2v t2 = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
-            x[e] = __builtin_fmaf((float)t2[0], kLog2e / 8.f, nlse4[e]);
-            x[e + 1] = __builtin_fmaf((float)t2[1], kLog2e / 8.f, nlse4[e + 1]);
+            if (MODE == kStatKfSeededFast) {
+              // ((t log2e - log2 E) / tau) - lse: E = -ln u in [6e-8, 16.7]
+              const float l0 = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(noise_uniform(row4[e], b_j)));
+              const float l1 = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(noise_uniform(row4[e + 1], b_j)));
+              x[e] = __builtin_fmaf(__builtin_fmaf((float)t2[0], kLog2e / 8.f, -l0), p.inv_tau, nlse4[e]);
+              x[e + 1] = __builtin_fmaf(__builtin_fmaf((float)t2[1], kLog2e / 8.f, -l1), p.inv_tau, nlse4[e + 1]);
+            } else {
+              x[e] = __builtin_fmaf((float)t2[0], kLog2e / 8.f, nlse4[e]);
+              x[e + 1] = __builtin_fmaf((float)t2[1], kLog2e / 8.f, nlse4[e + 1]);
+            }
           }
         } else {
 #pragma unroll
@@ -207,7 +217,9 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
           if (MODE == kStatCormRule) {
             best[e] = fmaxf(best[e], xv);
           } else {
-            const float pr = __builtin_amdgcn_exp2f(xv);
+            float pr = __builtin_amdgcn_exp2f(xv);
+            if (MODE == kStatKfSeededTau1)  // exp(t - lse) / E
+              pr *= __builtin_amdgcn_rcpf(-kLn2 * __builtin_amdgcn_logf(noise_uniform(row4[e], b_j)));
             if (MODE == kStatCormTensor) {
               best[e] = fmaxf(best[e], pr - er[mbk][4 * q4 + e] * (1.f - kCormSlack));
             } else {
@@ -225,7 +237,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
     for (int i = 0; i < 2 * KSTEPS; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, KFM ? 24 : 12, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, (KFM || KFP) ? 24 : 12, 0);
     }
   };
 
@@ -319,6 +331,12 @@ static hipError_t launch_td(const ColstatsKernelParams& p, bool causal, bool emu
   FT_CASE(C, E, kStatSum) FT_CASE(C, E, kStatSumSq) FT_CASE(C, E, kStatKfTensor) FT_CASE(C, E, kStatKfSeeded) \
   FT_CASE(C, E, kStatCormRule) FT_CASE(C, E, kStatCormTensor)
   FT_MODES(true, true) FT_MODES(true, false) FT_MODES(false, true) FT_MODES(false, false)
+  if constexpr (std::is_same<T, F16>::value) {  // packed KeyFormer modes: fp16 with reference rounding only
+    if (emu) {
+      FT_CASE(true, true, kStatKfSeededTau1) FT_CASE(false, true, kStatKfSeededTau1)
+      FT_CASE(true, true, kStatKfSeededFast) FT_CASE(false, true, kStatKfSeededFast)
+    }
+  }
 #undef FT_MODES
 #undef FT_CASE
   return hipErrorInvalidValue;

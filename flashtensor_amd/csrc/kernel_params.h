@@ -52,8 +52,15 @@ struct ColstatsKernelParams {
 };
 
 // what happens to a logit between the scaled QK^T and the softmax of the attention pass
-enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2, kKfSoftcap = 3 };
+// kKfSeededTau1 / kKfSeededFast: the seeded KeyFormer stream inside the packed fp16 path.  The perturbed
+// weight exp((t + g) / tau) with g = -ln E equals exp(t / tau) E^(-1/tau); the in-kernel E lies in
+// [6e-8, 16.7], so for tau >= 0.25 the plain softmax's running maximum also stabilises the perturbed sum
+// (exponent <= (6 + 24) / tau <= 120) and no second maximum is tracked; tau == 1 needs 1 / E only.
+enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2, kKfSoftcap = 3, kKfSeededTau1 = 4, kKfSeededFast = 5 };
 // kStatCormRule: thresholds 1 / (i + 1) per query row i; kStatCormTensor: thresholds read from a tensor
-enum StatMode { kStatSum = 0, kStatSumSq = 1, kStatKfTensor = 2, kStatKfSeeded = 3, kStatCormRule = 4, kStatCormTensor = 5 };
+enum StatMode {
+  kStatSum = 0, kStatSumSq = 1, kStatKfTensor = 2, kStatKfSeeded = 3, kStatCormRule = 4, kStatCormTensor = 5,
+  kStatKfSeededTau1 = 6, kStatKfSeededFast = 7  // seeded KeyFormer inside the packed fp16 path (see KfMode)
+};
 
 }  // namespace ft

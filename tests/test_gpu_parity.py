@@ -88,6 +88,37 @@ def test_keyformer_small(gpu, B, S, H, D, seed, tau):
   assert torch.allclose(ed, es, rtol=2e-6, atol=0)
 
 
+@pytest.mark.parametrize("tau", [0.2, 0.25, 0.5, 1.0, 4.0])
+def test_keyformer_seeded_paths(gpu, tau):
+  """tau == 1 and tau >= 0.25 take the packed path (no second running maximum), smaller tau the generic one;
+  long rows (several rescales of the running maximum), a rectangular problem and an unmasked one.  Two
+  checks: against the oracle on N(0,1) inputs, and - with logits 2.25 times larger, where one fp16 ulp of
+  QK^T (0.125 above 128) moves a dominant weight by several percent at small tau, so that only a loose
+  oracle comparison is meaningful - against the generic tensor-noise path fed the same noise."""
+  for (B, S, H, D, kv, causal, seed) in [(1, 1100, 2, 128, None, True, 31), (1, 96, 2, 64, 232, True, 32), (1, 160, 2, 128, None, False, 33)]:
+    (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed, kv_len=kv)
+    Skv = k.shape[1]
+    es = oracle.seeded_exp_rand(5 + seed, B, H, S, Skv)
+
+    def ref(qq, kk):
+      if causal:
+        return oracle.keyformer_forward(qq, kk, v, es, tau=tau)
+      scores = (torch.matmul(qq.transpose(1, 2), kk.transpose(1, 2).transpose(-2, -1)) / np.sqrt(D)).float()
+      return None, torch.softmax((scores - es.log()) / tau, -1).sum(2)
+
+    ref_o, ref_s = ref(q, k)
+    out, s = ops.keyformer(qd, kd, vd, None, tau=tau, seed=5 + seed, causal=causal)
+    if ref_o is not None:
+      check_o(out, ref_o)
+    check_score(s, ref_s, rel=SCORE_REL if tau >= 0.5 else 4e-3)
+    assert abs(s.sum().item() - B * H * S) < 1e-3 * B * H * S
+    out_s, s_s = ops.keyformer(qd * 1.5, kd * 1.5, vd, None, tau=tau, seed=5 + seed, causal=causal)
+    out_t, s_t = ops.keyformer(qd * 1.5, kd * 1.5, vd, es.to(gpu), tau=tau, causal=causal)
+    assert (out_s.float() - out_t.float()).abs().max().item() <= 4e-3   # packed and generic paths round P at different points
+    check_score(s_s, s_t.cpu(), rel=2e-5)
+    check_score(s_s, ref(q * 1.5, k * 1.5)[1], rel=5e-2)
+
+
 def test_rectangular_prefill_offset(gpu):
   # Sq < Skv: query i sees keys j <= i + (Skv - Sq)  (cases/kernels/attn.py:23)
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 96, 2, 128, seed=3, kv_len=232)
