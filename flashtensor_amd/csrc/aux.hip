@@ -8,9 +8,12 @@
 
 namespace ft {
 
-// One workgroup sorts one row: (score, index) pairs packed into 64-bit keys whose unsigned order is
-// "score descending, index ascending", bitonic sort in LDS, first k indices written out.
-constexpr int kTopkThreads = 1024;
+// One workgroup of NT threads sorts one row: (score, index) pairs packed into 64-bit keys whose unsigned
+// order is "score descending, index ascending", bitonic network over N = NT E keys, first k indices written
+// out.  Thread t keeps keys t E .. t E + E - 1 in registers, so a compare-exchange at distance < E stays inside
+// the thread, one at distance < 64 E is a lane exchange inside the wave (no barrier), and only the few
+// steps at distance >= 64 E go through LDS (3 with 256 threads, 6 with 512) instead of one barrier per
+// network step.  E <= 16 keeps the fully unrolled network's keys in registers.
 
 __device__ __forceinline__ uint32_t float_order_desc(float x) {
   uint32_t u = __builtin_bit_cast(uint32_t, x);
@@ -18,48 +21,78 @@ __device__ __forceinline__ uint32_t float_order_desc(float x) {
   return ~u;                                       // flipped: larger scores first
 }
 
-__global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float* __restrict__ score, int S, int N /*pow2 >= S*/, int k,
-                                                            int64_t* __restrict__ idx) {
-  extern __shared__ __align__(16) char smem_raw[];
-  uint64_t* keys = reinterpret_cast<uint64_t*>(smem_raw);
+__device__ __forceinline__ uint64_t lane_xor_u64(uint64_t v, int mask) {
+  const uint32_t lo = __shfl_xor((uint32_t)v, mask), hi = __shfl_xor((uint32_t)(v >> 32), mask);
+  return ((uint64_t)hi << 32) | lo;
+}
+
+template <int E, int NT>
+__global__ void __launch_bounds__(NT) topk_kernel(const float* __restrict__ score, int S, int k, int64_t* __restrict__ idx) {
+  constexpr int N = NT * E;
+  __shared__ uint64_t xch[N];  // slot-major: key e of thread t at [e * NT + t]
+  const int t = threadIdx.x;
   const float* row = score + (int64_t)blockIdx.x * S;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) {
-    uint64_t key = ~0ull;  // padding sorts last
-    if (i < S) key = ((uint64_t)float_order_desc(row[i]) << 32) | (uint32_t)i;
-    keys[i] = key;
+  uint64_t key[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = t * E + e;
+    key[e] = i < S ? (((uint64_t)float_order_desc(row[i]) << 32) | (uint32_t)i) : ~0ull;  // padding sorts last
   }
-  __syncthreads();
+#pragma unroll
   for (int size = 2; size <= N; size <<= 1) {
+#pragma unroll
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int t = threadIdx.x; t < N / 2; t += blockDim.x) {
-        const int lo = 2 * t - (t & (stride - 1));
-        const int hi = lo + stride;
-        const bool ascending = (lo & size) == 0;
-        const uint64_t a = keys[lo], b = keys[hi];
-        if ((a > b) == ascending) {
-          keys[lo] = b;
-          keys[hi] = a;
+      if (stride < E) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          if ((e & stride) == 0) {
+            const bool up = ((t * E + e) & size) == 0;
+            const uint64_t a = key[e], b = key[e | stride];
+            const bool swap = (a > b) == up;
+            key[e] = swap ? b : a;
+            key[e | stride] = swap ? a : b;
+          }
         }
+      } else {
+        const int m = stride / E;  // partner thread t ^ m holds the partner of every key of this thread
+        const bool lower = (t & m) == 0;
+        if (m >= 64) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) xch[e * NT + t] = key[e];
+          __syncthreads();
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const uint64_t a = key[e];
+          const uint64_t b = m >= 64 ? xch[e * NT + (t ^ m)] : lane_xor_u64(a, m);
+          const bool up = ((t * E + e) & size) == 0;
+          const bool want_min = lower == up;
+          key[e] = ((a < b) == want_min) ? a : b;
+        }
+        if (m >= 64) __syncthreads();
       }
-      __syncthreads();
     }
   }
   int64_t* out = idx + (int64_t)blockIdx.x * k;
-  for (int i = threadIdx.x; i < k; i += blockDim.x) out[i] = (int64_t)(uint32_t)keys[i];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = t * E + e;
+    if (i < k) out[i] = (int64_t)(uint32_t)key[e];
+  }
 }
 
 hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* idx, hipStream_t s) {
-  int N = 2;
-  while (N < S) N <<= 1;
-  const int lds = N * 8;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(topk_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 8192 * 8);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
-  const int threads = N / 2 < kTopkThreads ? (N / 2 < 64 ? 64 : N / 2) : kTopkThreads;
-  hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows), dim3(threads), lds, s, score, S, N, k, idx);
+  const dim3 grid((unsigned)rows);
+  if (S <= 512)
+    hipLaunchKernelGGL((topk_kernel<2, 256>), grid, dim3(256), 0, s, score, S, k, idx);
+  else if (S <= 1024)
+    hipLaunchKernelGGL((topk_kernel<4, 256>), grid, dim3(256), 0, s, score, S, k, idx);
+  else if (S <= 2048)
+    hipLaunchKernelGGL((topk_kernel<8, 256>), grid, dim3(256), 0, s, score, S, k, idx);
+  else if (S <= 4096)
+    hipLaunchKernelGGL((topk_kernel<16, 256>), grid, dim3(256), 0, s, score, S, k, idx);
+  else
+    hipLaunchKernelGGL((topk_kernel<16, 512>), grid, dim3(512), 0, s, score, S, k, idx);
   return hipGetLastError();
 }
 

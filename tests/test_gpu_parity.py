@@ -233,6 +233,15 @@ def test_topk_matches_torch_and_orders_ties(gpu):
   assert ops.topk(t, 4).tolist() == [[1, 2, 4, 0]]  # ties: lower index first
   s3 = torch.randn(3, 1000, generator=g).to(gpu)    # not a power of two
   assert torch.equal(ops.topk(s3, 125), torch.topk(s3, 125).indices)
+  # every network size (512 .. 8192 keys), full sorts, k == 1, rows of equal values, infinities
+  for S in (1, 7, 64, 512, 513, 1024, 3000, 4096, 4097, 8192):
+    x = torch.randn(4, S, generator=g).to(gpu)
+    for k in sorted({1, max(1, S // 8), S}):
+      assert torch.equal(ops.topk(x, k), torch.topk(x, k).indices), (S, k)
+  flat = torch.zeros(2, 700, device=gpu)
+  assert torch.equal(ops.topk(flat, 700), torch.arange(700, device=gpu).expand(2, 700))
+  spec = torch.tensor([[0.0, float("inf"), -float("inf"), 2.0, -0.0, 1e-40]], device=gpu)
+  assert ops.topk(spec, 6).tolist()[0][:2] == [1, 3] and ops.topk(spec, 6).tolist()[0][-1] == 2
 
 
 # ------------------------------------------------------------------ builder / case modules
