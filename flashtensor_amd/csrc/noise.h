@@ -5,10 +5,12 @@
 // Here element (bh, i, j) of that tensor is a pure function of (seed, bh, i, j), so the two passes of
 // the fused kernels regenerate it instead of reading 4 bytes per logit from HBM:
 //   k0 = mix(seed_lo ^ mix(bh + 0x9E3779B9)),  k1 = mix(seed_hi ^ k0 ^ 0x85EBCA6B)
-//   a_i = mix(i ^ k0),  b_j = mix(j ^ k1),  x = mix(a_i + b_j)
+//   a_i = mix(i ^ k0),  b_j = mix(j ^ k1) | 1,  x = a_i * b_j,  x ^= x >> 16
 //   u = ((x >> 9) + 0.5) * 2^-23  in (0,1);   E = -ln(u) ~ Exp(1);   gumbel = -ln(E)
-// with mix = the lowbias32 integer finaliser.  a_i and b_j are per-row / per-column values, so the
-// per-element cost is one add and one mix.
+// with mix = the lowbias32 integer finaliser.  a_i and b_j are fully mixed per-row / per-column values, so
+// the per-element cost is one 32-bit multiply and one xor-shift; the top 23 bits of the product of two
+// mixed words pass the uniformity, neighbour-correlation, pair and 2x2 mixed-difference tests that a
+// one-round mix of the sum a_i + b_j fails (its additive structure survives one round).
 #pragma once
 #include <stdint.h>
 
@@ -41,11 +43,12 @@ FT_HD NoiseKeys noise_keys(uint64_t seed, uint32_t bh) {
 }
 
 FT_HD uint32_t noise_row(NoiseKeys k, uint32_t i) { return mix32(i ^ k.k0); }
-FT_HD uint32_t noise_col(NoiseKeys k, uint32_t j) { return mix32(j ^ k.k1); }
+FT_HD uint32_t noise_col(NoiseKeys k, uint32_t j) { return mix32(j ^ k.k1) | 1u; }
 
 // u in (0,1) from the row and column terms; exact in fp32.
 FT_HD float noise_uniform(uint32_t a_i, uint32_t b_j) {
-  uint32_t x = mix32(a_i + b_j);
+  uint32_t x = a_i * b_j;
+  x ^= x >> 16;
   return (float)(x >> 9) * 1.1920928955078125e-07f + 5.9604644775390625e-08f;
 }
 

@@ -12,7 +12,7 @@ defines its own stream, and this module materialises exactly the tensor the kern
 Stream definition (all arithmetic mod 2**32):
     lowbias32(x): x ^= x>>16; x *= 0x7feb352d; x ^= x>>15; x *= 0x846ca68b; x ^= x>>16
     k0 = lowbias32(seed_lo ^ lowbias32(bh + 0x9E3779B9));  k1 = lowbias32(seed_hi ^ k0 ^ 0x85EBCA6B)
-    a_i = lowbias32(i ^ k0);  b_j = lowbias32(j ^ k1);  x_ij = lowbias32(a_i + b_j)
+    a_i = lowbias32(i ^ k0);  b_j = lowbias32(j ^ k1) | 1;  x_ij = a_i * b_j;  x_ij ^= x_ij >> 16
     u_ij = ((x_ij >> 9) + 0.5) * 2**-23        in (0,1), exact in fp32
     E_ij = -ln(u_ij)                            ~ Exp(1);  g_ij = -ln(E_ij) ~ Gumbel(0,1)
 with bh = b*H + h, i the query row and j the key column.
@@ -46,8 +46,10 @@ def noise_u32(seed, bh, rows, cols):
   """x_ij for one (b,h) pair: rows, cols are 1-D integer arrays -> uint32 [len(rows), len(cols)]."""
   k0, k1 = _keys(seed, bh)
   a = lowbias32(np.asarray(rows, dtype=np.uint64) ^ k0.astype(np.uint64)).astype(np.uint64)
-  b = lowbias32(np.asarray(cols, dtype=np.uint64) ^ k1.astype(np.uint64)).astype(np.uint64)
-  return lowbias32((a[:, None] + b[None, :]) & _M)
+  b = lowbias32(np.asarray(cols, dtype=np.uint64) ^ k1.astype(np.uint64)).astype(np.uint64) | np.uint64(1)
+  x = (a[:, None] * b[None, :]) & _M
+  x ^= x >> np.uint64(16)
+  return x.astype(np.uint32)
 
 
 def seeded_exp_rand(seed, B, H, Sq, Skv, row_offset=0):

@@ -244,6 +244,28 @@ def test_lowbias32_known_answers():
   got = oracle.lowbias32(np.array(xs, dtype=np.uint64))
   assert [int(g) for g in got] == [ref(x) for x in xs]
   assert int(oracle.lowbias32(0)) == 0 and len(set(int(g) for g in got)) == len(xs)
+  # the element combiner, by hand with Python integers: seed 7, head 3, row 11, column 5
+  seed, bh, i, j = 7, 3, 11, 5
+  k0 = ref((seed & 0xFFFFFFFF) ^ ref(bh + 0x9E3779B9)); k1 = ref((seed >> 32) ^ k0 ^ 0x85EBCA6B)
+  a, b = ref(i ^ k0), ref(j ^ k1) | 1
+  x = (a * b) & 0xFFFFFFFF; x ^= x >> 16
+  assert int(oracle.noise_u32(seed, bh, [i], [j])[0, 0]) == x
+  E = oracle.seeded_exp_rand(seed, 1, 4, 12, 6)[0, 3, 11, 5].item()
+  assert abs(E - -math.log(((x >> 9) + 0.5) * 2.0 ** -23)) < 1e-6 * E
+
+
+def test_noise_stream_has_no_lattice_structure():
+  # sums and differences over 2x2 minors: u_ij - u_ij' - u_i'j + u_i'j' (mod 1) is uniform for independent
+  # draws; a generator that only adds a row term and a column term before a weak mix fails this badly
+  from scipy import stats
+  x = oracle.noise_u32(99, 0, np.arange(768), np.arange(768))
+  u = ((x >> np.uint32(9)).astype(np.float64) + 0.5) * 2.0 ** -23
+  d = (u[:-1, :-1] - u[:-1, 1:] - u[1:, :-1] + u[1:, 1:] + 0.5) % 1.0
+  assert stats.chisquare(np.bincount((d.flatten() * 256).astype(int) % 256, minlength=256)).pvalue > 1e-4
+  pairs = np.bincount((u[:, :-1].flatten() * 64).astype(int) * 64 + (u[:, 1:].flatten() * 64).astype(int), minlength=4096)
+  assert stats.chisquare(pairs).pvalue > 1e-4
+  pairs = np.bincount((u[:-1].flatten() * 64).astype(int) * 64 + (u[1:].flatten() * 64).astype(int), minlength=4096)
+  assert stats.chisquare(pairs).pvalue > 1e-4
 
 
 # ------------------------------------------------------------------ SnapKV, CoRM, Gemma2
