@@ -42,7 +42,9 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
   constexpr bool kIsF16 = __is_same(typename T::elem, _Float16);
   constexpr bool kKfFast = KF == kKfSeededTau1 || KF == kKfSeededFast;           // seeded noise inside the packed path
   constexpr bool kSeeded = KF == kKfSeeded || kKfFast;
-  constexpr bool kFastMasked = kIsF16 && EMU && (KF == kKfNone || kKfFast);  // variants served by the packed-fp16 softmax
+  // variants served by the pipelined fast path: fp16 plain softmax with either treatment of the logits, and
+  // the packed seeded KeyFormer modes
+  constexpr bool kFastMasked = kIsF16 && ((EMU && kKfFast) || KF == kKfNone);
   static_assert(!kKfFast || (kIsF16 && EMU), "the packed KeyFormer modes exist for fp16 with reference rounding only");
   // Software pipeline across tiles: the QK^T MFMAs of tile it+1 are issued in the same iteration as the
   // softmax (VALU) and PV MFMAs of tile it, so the matrix and vector pipes overlap inside one wave.
@@ -218,7 +220,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
     }
     float amax = __builtin_fmaxf(max3(m4[0], m4[1], m4[2]), m4[3]);
     amax = __builtin_fmaxf(amax, xchg32(amax));
-    rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
+    if (EMU)
+      rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
+    else
+      rescale(amax * p.logit_mul);  // logit_mul = log2e / sqrt(D) when the logits stay in fp32
   };
   // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.
   auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0, int buf) {
@@ -236,16 +241,19 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       const int mbk = blk >> 1, rb = (blk & 1) * 8;
       half2v t2[4];
       float x[8];
+      if constexpr (EMU) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float2v a2 = {s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]};
-        const half2v h2 = __builtin_convertvector(a2, half2v);  // QK^T is an fp16 tensor in the reference
-        // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
-        t2[i] = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
+        for (int i = 0; i < 4; ++i) {
+          const float2v a2 = {s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]};
+          const half2v h2 = __builtin_convertvector(a2, half2v);  // QK^T is an fp16 tensor in the reference
+          // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
+          t2[i] = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        x[i] = __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m);
+        x[i] = EMU ? __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m)
+                   : __builtin_fmaf(s[mbk][rb + i], p.logit_mul, neg_m);
         if (MASKED) {
           const int jl = 32 * mbk + 8 * ((rb + i) >> 2) + ((rb + i) & 3);
           x[i] = (jl > lim) ? NEG_INF : x[i];

@@ -25,10 +25,11 @@ constexpr int kColBK = 128;  // keys per workgroup
 constexpr int kColBQ = 64;   // query rows per tile
 constexpr int kColThreads = 256;
 
-// waves per SIMD the register budget is sized for: the packed-fp16 sum / sum-of-squares variants fit three
+// waves per SIMD the register budget is sized for: the sum / sum-of-squares variants with a short logit chain
+// (packed fp16 rounding, or logits kept in fp32) fit three
 template <typename T, bool EMU, int MODE>
 constexpr int colstats_waves_per_simd() {
-  return (__is_same(typename T::elem, _Float16) && EMU && (MODE == kStatSum || MODE == kStatSumSq)) ? 3 : 2;
+  return ((__is_same(typename T::elem, _Float16) || !EMU) && (MODE == kStatSum || MODE == kStatSumSq)) ? 3 : 2;
 }
 
 template <typename T, int D, bool CAUSAL, bool EMU, int MODE>
@@ -43,6 +44,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   constexpr bool kSeeded = MODE == kStatKfSeeded || KFP;
   constexpr bool CORM = (MODE == kStatCormRule || MODE == kStatCormTensor);
   constexpr bool kPacked = __is_same(typename T::elem, _Float16) && EMU;  // packed-fp16 rounding chain
+  constexpr bool kPlainF32 = !EMU;                                        // logits stay in fp32: one fma per element
   // one LDS object per buffer: reads of one do not wait for the direct-to-LDS loads in flight into the other
   __shared__ __align__(16) char ldsQ0[TILE_BYTES];
   __shared__ __align__(16) char ldsQ1[TILE_BYTES];
@@ -168,7 +170,10 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
         uint4v row4 = {0, 0, 0, 0};
         if (kSeeded) row4 = *reinterpret_cast<const uint4v*>(ldsRow + buf * BQ + il0 + 4 * g);
         float x[4];
-        if (kPacked && !KFM) {
+        if (kPlainF32 && !KFM && !KFP) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[e] = __builtin_fmaf(s[mbk][4 * q4 + e], p.logit_mul, nlse4[e]);
+        } else if (kPacked && !KFM) {
 #pragma unroll
           for (int e = 0; e < 4; e += 2) {
             const float2v a2 = {s[mbk][4 * q4 + e], s[mbk][4 * q4 + e + 1]};
