@@ -401,6 +401,46 @@ def test_next_cases_at_reference_default_shape(gpu):
   assert torch.equal(f(qd, kd, vd)[1], s)
 
 
+# ------------------------------------------------------------------ few heads, long rows (fewer workgroups than CUs)
+
+FEW_HEADS = [(1, 512, 2, 128, 40), (1, 1000, 3, 128, 41), (1, 640, 2, 64, 42), (2, 777, 2, 128, 43), (1, 2048, 1, 128, 44), (1, 1537, 4, 64, 45)]
+
+
+@pytest.mark.parametrize("B,S,H,D,seed", FEW_HEADS)
+def test_few_heads_long_rows(gpu, B, S, H, D, seed):
+  """Problems that leave most CUs idle: many key tiles per query block, several rescales of the running
+  maximum, ragged tails; O, and through the normaliser the H2O / RoCo scores."""
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  ref_o, r1, r2 = oracle.roco_forward(q, k, v)
+  check_o(ops.attn(qd, kd, vd), ref_o)
+  out, s1, s2 = ops.roco(qd, kd, vd)
+  check_o(out, ref_o); check_score(s1, r1); check_score(s2, r2)
+  # larger logits: the running maximum moves several times
+  ref_big = oracle.attn_forward(q * 2, k * 2, v)
+  check_o(ops.attn(qd * 2, kd * 2, vd), ref_big)
+
+
+def test_few_heads_rectangular_noncausal_grouped(gpu):
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 96, 2, 128, seed=46, kv_len=700)
+  ref_o, r1 = oracle.h2o_forward(q, k, v)
+  out, s1 = ops.h2o(qd, kd, vd)
+  check_o(out, ref_o); check_score(s1, r1)
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 100, 2, 64, seed=47, kv_len=600)
+  p = torch.softmax((torch.matmul(q.transpose(1, 2), k.transpose(1, 2).transpose(-2, -1)) / np.sqrt(64)).float(), -1)
+  out, s1 = ops.h2o(qd, kd, vd, causal=False)
+  check_o(out, torch.matmul(p.half(), v.transpose(1, 2)).transpose(1, 2)); check_score(s1, p.sum(2))
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 900, 4, 128, seed=48)
+  kg, vg = kd[:, :, :2].contiguous(), vd[:, :, :2].contiguous()
+  out_g = ops.attn(qd, kg, vg)
+  ref = oracle.attn_forward(q, k[:, :, :2].repeat_interleave(2, dim=2), v[:, :, :2].repeat_interleave(2, dim=2))
+  check_o(out_g, ref)
+  # the same problem replicated over many heads (another workgroup-to-CU mapping) gives the same rows
+  qr, kr, vr = (t.repeat(1, 1, 16, 1) for t in (qd, kd, vd))   # 64 heads x 8 blocks = 512 workgroups
+  out_small = ops.attn(qd, kd, vd)
+  out_big = ops.attn(qr, kr, vr)[:, :, :4]
+  assert (out_small.float() - out_big.float()).abs().max().item() <= 2e-3
+
+
 # ------------------------------------------------------------------ grouped queries, 2-D harness form
 
 @pytest.mark.parametrize("S,Skv,H,Hkv,D,masked", [(128, 128, 4, 2, 128, True), (200, 200, 8, 2, 64, True), (96, 232, 4, 1, 128, True),
