@@ -693,7 +693,9 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
       const int r = j * (64 / LPR) + lane / LPR;
       const int c = lane % LPR;
       const uint4v val = *reinterpret_cast<const uint4v*>(ost + r * OROW + c * 16);
-      if (t0 + r < p.S) *reinterpret_cast<uint4v*>(obase + (int64_t)(t0 + r) * orow_bytes + c * 16) = val;
+      // streamed out once and not read again here: non-temporal, so that the lines do not linger dirty in
+      // the caches and get written back under the next kernel's reads
+      if (t0 + r < p.S) __builtin_nontemporal_store(val, reinterpret_cast<uint4v*>(obase + (int64_t)(t0 + r) * orow_bytes + c * 16));
     }
     wave_lds_order();
   };
