@@ -85,6 +85,17 @@ def per_config_table(dev):
   lin_flops, lin_bytes = 2 * 2.0 * 8 * 16 * 8192 * 64 * 64, 4.0 * 8 * 16 * 8192 * 64 * 2
   add("5 ea", "B8 H16 S8192 D64", lambda: ops.ea(q, k, v), lin_flops, lin_bytes)
   add("5 sima", "B8 H16 S8192 D64", lambda: ops.sima(q, k, v), lin_flops, lin_bytes)
+  del q, k, v
+  # the whole function of bench/ea.mlir / bench/sima.mlir: hipBLASLt projections around the core (C = 1024)
+  C, M = 16 * 64, 8 * 8192
+  x = torch.randn(8, 8192, C, dtype=torch.float16, device=dev)
+  wq = (torch.randn(3 * C, C, device=dev) / C ** 0.5).half()
+  wo = (torch.randn(C, C, device=dev) / C ** 0.5).half()
+  bq, bo = torch.zeros(3 * C, dtype=torch.float16, device=dev), torch.zeros(C, dtype=torch.float16, device=dev)
+  blk_flops = lin_flops + 2.0 * M * (3 * C * C + C * C)
+  blk_bytes = (2.0 * M * C + 4 * C * C + 4 * C) * 2  # x in, y out, the weights and biases once
+  add("5b ea block (projections + core)", "B8 S8192 C1024 H16", lambda: ops.ea_block(x, wq, bq, wo, bo, 16), blk_flops, blk_bytes)
+  add("5b sima block", "B8 S8192 C1024 H16", lambda: ops.sima_block(x, wq, bq, wo, bo, 16, normalize_q=False), blk_flops, blk_bytes)
   return rows
 
 

@@ -12,12 +12,12 @@ FT_OK, FT_EINVAL, FT_EUNSUPPORTED, FT_ELAUNCH, FT_EWORKSPACE = 0, -1, -2, -3, -4
 FT_F16, FT_BF16, FT_F32 = 0, 1, 2
 FT_CAUSAL, FT_FAST_LOGITS = 1, 2
 FT_OP_ATTN, FT_OP_COLSTATS, FT_OP_KEYFORMER, FT_OP_EA, FT_OP_SIMA, FT_OP_CORM = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # every symbol include/ft_abi.h declares
 EXPORTS = ("ft_abi_version", "ft_last_error", "ft_workspace_bytes", "ft_attn_fwd", "ft_attn_colstats_fwd",
            "ft_keyformer_fwd", "ft_attn_softcap_fwd", "ft_corm_fwd", "ft_avgpool1d", "ft_linattn_fwd", "ft_topk",
-           "ft_noise_exp_fill", "ft_noise_exp_fill_host")
+           "ft_noise_exp_fill", "ft_noise_exp_fill_host", "ft_linattn_block_workspace_bytes", "ft_linattn_block_fwd")
 
 
 class FtStrides(ctypes.Structure):
@@ -29,6 +29,13 @@ class FtAttnArgs(ctypes.Structure):
               ("sq", FtStrides), ("sk", FtStrides), ("sv", FtStrides), ("so", FtStrides),
               ("B", ctypes.c_int32), ("H", ctypes.c_int32), ("Sq", ctypes.c_int32), ("Skv", ctypes.c_int32),
               ("D", ctypes.c_int32), ("dtype", ctypes.c_int32), ("flags", ctypes.c_uint32), ("Hkv", ctypes.c_int32)]
+
+
+class FtLinBlockArgs(ctypes.Structure):
+  _fields_ = [("x", ctypes.c_void_p), ("w_qkv", ctypes.c_void_p), ("b_qkv", ctypes.c_void_p), ("w_out", ctypes.c_void_p),
+              ("b_out", ctypes.c_void_p), ("y", ctypes.c_void_p),
+              ("B", ctypes.c_int32), ("S", ctypes.c_int32), ("H", ctypes.c_int32), ("D", ctypes.c_int32),
+              ("dtype", ctypes.c_int32)]
 
 
 class FtNoise(ctypes.Structure):
@@ -84,6 +91,11 @@ def load():
   lib.ft_noise_exp_fill.argtypes = [f32p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64, vp]
   lib.ft_noise_exp_fill_host.restype = ctypes.c_int
   lib.ft_noise_exp_fill_host.argtypes = [f32p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+  block_p = ctypes.POINTER(FtLinBlockArgs)
+  lib.ft_linattn_block_workspace_bytes.restype = ctypes.c_size_t
+  lib.ft_linattn_block_workspace_bytes.argtypes = [block_p, ctypes.c_int]
+  lib.ft_linattn_block_fwd.restype = ctypes.c_int
+  lib.ft_linattn_block_fwd.argtypes = [block_p, ctypes.c_int, ctypes.c_int, vp, ctypes.c_size_t, vp]
   if lib.ft_abi_version() != ABI_VERSION:
     raise ImportError(f"ABI version mismatch: library {lib.ft_abi_version()}, binding {ABI_VERSION}")
   _lib = lib

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libflashtensor_hip.so")
-SOURCES = ["abi.hip", "attn_fwd.hip", "colstats.hip", "linattn.hip", "aux.hip"]
+SOURCES = ["abi.hip", "attn_fwd.hip", "colstats.hip", "linattn.hip", "aux.hip", "linblock.hip"]
 HEADERS = ["device_common.hpp", "kernel_params.h", "noise.h", os.path.join("..", "..", "include", "ft_abi.h")]
 # packed fp32 VALU ops are disabled on purpose: some forms have produced wrong results on this hardware
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

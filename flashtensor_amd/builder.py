@@ -36,6 +36,13 @@ class HipBuilder(Builder):
     if not self.check_before_run:
       return model.forward
     head_num, head_dim = model.head_num, model.head_dim
+    if hasattr(model, "check_args"):  # cases whose arguments are not q, k, v
+
+      def g(*args):
+        model.check_args(*args)
+        return model.forward(*args)
+
+      return g
 
     def f(*args):
       for i, arg in enumerate(args[:3]):

@@ -39,6 +39,21 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+}  // namespace
+
+namespace ft {
+// ft_last_error() for the translation units that hold entry points of their own
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+}  // namespace ft
+
+namespace {
+
 int hip_fail(hipError_t e, const char* what) {
   return fail(FT_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
 }

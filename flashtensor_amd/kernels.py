@@ -191,8 +191,53 @@ class SimA(EA):
     return ops.sima(q, k, v, normalize_q=self.normalize_q)
 
 
+class EABlock:
+  """The function of bench/ea.mlir:2-23 with its five arguments in order: x, the q/k/v Linear's weight and
+  bias, the output Linear's weight and bias."""
+  output = ["out"]
+
+  def __init__(self, head_num=16, head_dim=64):
+    self.head_num = head_num
+    self.head_dim = head_dim
+    self.hidden_size = head_num * head_dim
+
+  def __call__(self, *args):
+    return self.forward(*args)
+
+  def eval(self):
+    return self
+
+  def check_args(self, x, *rest):
+    if x.dim() != 3 or x.shape[2] != self.hidden_size:
+      raise RuntimeError(f"arg 0 need shape (B, S, {self.hidden_size}) but got {tuple(x.shape)}")
+
+  def forward(self, x, w_qkv, b_qkv, w_out, b_out):
+    return ops.ea_block(x, w_qkv, b_qkv, w_out, b_out, self.head_num)
+
+  def prepare(self, batch_size=8, q_len=8192, kv_len=None, dtype=torch.float16, device=None):
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    C = self.hidden_size
+    x = torch.randn(batch_size, q_len, C, dtype=dtype, device=device)
+    w_qkv = (torch.randn(3 * C, C, dtype=torch.float32, device=device) / C ** 0.5).to(dtype)
+    b_qkv = (0.1 * torch.randn(3 * C, dtype=torch.float32, device=device)).to(dtype)
+    w_out = (torch.randn(C, C, dtype=torch.float32, device=device) / C ** 0.5).to(dtype)
+    b_out = (0.1 * torch.randn(C, dtype=torch.float32, device=device)).to(dtype)
+    return {"input": {"x": x, "w_qkv": w_qkv, "b_qkv": b_qkv, "w_out": w_out, "b_out": b_out}, "output": self.output}
+
+
+class SimABlock(EABlock):
+  """The function of bench/sima.mlir:2-23."""
+
+  def __init__(self, head_num=16, head_dim=64, normalize_q=True):
+    super().__init__(head_num, head_dim)
+    self.normalize_q = normalize_q
+
+  def forward(self, x, w_qkv, b_qkv, w_out, b_out):
+    return ops.sima_block(x, w_qkv, b_qkv, w_out, b_out, self.head_num, normalize_q=self.normalize_q)
+
+
 CASES = {"attn": Attn, "h2o": H2O, "kf": KeyFormer, "roco": RoCo, "snapkv": SnapKV, "corm": Corm, "gemma2": Gemma2,
-         "ea": EA, "sima": SimA}
+         "ea": EA, "sima": SimA, "ea_block": EABlock, "sima_block": SimABlock}
 
 
 def get_model(name="attn", **kw):

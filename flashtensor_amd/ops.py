@@ -201,6 +201,49 @@ def sima(q, k, v, normalize_q=True, out_dtype=None):
   return _linattn(q, k, v, _lib.FT_OP_SIMA, normalize_q, out_dtype)
 
 
+def _linattn_block(x, w_qkv, b_qkv, w_out, b_out, head_num, kind, normalize_q):
+  tensors = [("x", x), ("w_qkv", w_qkv), ("b_qkv", b_qkv), ("w_out", w_out), ("b_out", b_out)]
+  for i, (name, t) in enumerate(tensors):
+    if t is None and name.startswith("b_"):
+      continue
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+      raise RuntimeError(f"arg {i} ({name}) need a GPU tensor")
+    if t.dtype != x.dtype:
+      raise RuntimeError(f"arg {i} ({name}) need {x.dtype} but got {t.dtype}")
+  if x.dim() != 3 or x.shape[2] % head_num:
+    raise ValueError(f"x need [B,S,C] with C a multiple of head_num={head_num} but got {tuple(x.shape)}")
+  B, S, C = x.shape
+  if tuple(w_qkv.shape) != (3 * C, C) or tuple(w_out.shape) != (C, C):
+    raise ValueError(f"weights need [{3 * C},{C}] and [{C},{C}] but got {tuple(w_qkv.shape)} and {tuple(w_out.shape)}")
+  if (b_qkv is not None and tuple(b_qkv.shape) != (3 * C,)) or (b_out is not None and tuple(b_out.shape) != (C,)):
+    raise ValueError(f"biases need [{3 * C}] and [{C}]")
+  lib = _lib.load()
+  x, w_qkv, w_out = x.contiguous(), w_qkv.contiguous(), w_out.contiguous()
+  b_qkv = None if b_qkv is None else b_qkv.contiguous()
+  b_out = None if b_out is None else b_out.contiguous()
+  y = torch.empty_like(x)
+  dt = {torch.float16: _lib.FT_F16, torch.bfloat16: _lib.FT_BF16}.get(x.dtype, _lib.FT_F32)
+  a = _lib.FtLinBlockArgs(x.data_ptr(), w_qkv.data_ptr(), None if b_qkv is None else b_qkv.data_ptr(), w_out.data_ptr(),
+                          None if b_out is None else b_out.data_ptr(), y.data_ptr(), B, S, head_num, C // head_num, dt)
+  nbytes = lib.ft_linattn_block_workspace_bytes(ctypes.byref(a), kind)
+  if nbytes == 0:
+    _lib.check(_lib.FT_EUNSUPPORTED)
+  ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+  _lib.check(lib.ft_linattn_block_fwd(ctypes.byref(a), kind, int(bool(normalize_q)), ws.data_ptr(), nbytes, _stream(x)))
+  return y
+
+
+def ea_block(x, w_qkv, b_qkv, w_out, b_out, head_num):
+  """The whole function of bench/ea.mlir:2-23: q/k/v Linear, split into heads, EA core, output Linear.
+  x [B,S,C], w_qkv [3C,C], b_qkv [3C], w_out [C,C], b_out [C] -> [B,S,C]."""
+  return _linattn_block(x, w_qkv, b_qkv, w_out, b_out, head_num, _lib.FT_OP_EA, True)
+
+
+def sima_block(x, w_qkv, b_qkv, w_out, b_out, head_num, normalize_q=True):
+  """The whole function of bench/sima.mlir:2-23 (normalize_q as for `sima`)."""
+  return _linattn_block(x, w_qkv, b_qkv, w_out, b_out, head_num, _lib.FT_OP_SIMA, normalize_q)
+
+
 def topk(score, k):
   """Indices [..., k] (int64) of the k largest entries along the last axis, descending."""
   if score.dtype != torch.float32 or not score.is_cuda:

@@ -34,18 +34,24 @@ def build(args, device):
     gb = (2 * q.numel() + k.numel() + v.numel()) * esz / 1e9
     return model.forward, [q, k, v], gflop, gb
   hyper = {}
-  if args.model_name in ("ea", "sima"):
+  linear = args.model_name in ("ea", "sima", "ea_block", "sima_block")
+  block = args.model_name.endswith("_block")
+  if linear:
     head_num, head_dim = args.head_num or 16, args.head_dim or 64
   else:
     head_num, head_dim = args.head_num or 32, args.head_dim or 128
-  hyper.update(kv_head_num=head_num, head_num=head_num, head_dim=head_dim)
+  hyper.update(head_num=head_num, head_dim=head_dim)
+  if not block:
+    hyper.update(kv_head_num=head_num)
   f = HipBuilder(args.model_name, **hyper).build_callable()
   model = kernels.get_model(args.model_name, **hyper)
   inout = model.prepare(batch_size=args.batch_size, q_len=args.q_len, kv_len=args.kv_len, dtype=dtype, device=device)
   inputs = list(inout["input"].values())
   B, S, Skv = args.batch_size, args.q_len, args.kv_len
-  if args.model_name in ("ea", "sima"):
+  if linear:
     gflop = 4.0 * B * head_num * S * head_dim * head_dim / 1e9
+    if block:  # + the q/k/v and output projections, 2 M (3 C C + C C)
+      gflop += 8.0 * B * S * (head_num * head_dim) ** 2 / 1e9
   else:
     gflop = 2.0 * B * head_num * S * Skv * head_dim / 1e9  # two causal contractions
   gb = 4.0 * B * S * head_num * head_dim * esz / 1e9

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FT_ABI_VERSION 2
+#define FT_ABI_VERSION 3
 
 enum FtStatus {
   FT_OK = 0,
@@ -120,6 +120,30 @@ int ft_avgpool1d(const float* src, int64_t rows, int32_t S, int32_t kernel, floa
  * out_dtype: FtDtype of o (FT_F16/FT_BF16 = a->dtype, or FT_F32). */
 int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/* The whole block of bench/ea.mlir:2-23 / bench/sima.mlir:2-23 around the core: x [B,S,C] with C = H*D,
+ * qkv = x w_qkv^T + b_qkv (w_qkv [3C,C] row-major as in a Linear, :3-5), split into q, k, v and into heads
+ * (:6-12), the core (:13-17), y = core w_out^T + b_out (w_out [C,C], :20-22).  All tensors 16-bit and
+ * contiguous; biases may be NULL.  The two projections are hipBLASLt GEMMs (fp32 accumulation, bias added
+ * before the one rounding to 16 bits); q/k/v and the core's result live in the workspace as 16-bit tensors. */
+typedef struct FtLinBlockArgs {
+  const void* x;
+  const void* w_qkv;
+  const void* b_qkv;
+  const void* w_out;
+  const void* b_out;
+  void* y;
+  int32_t B, S, H, D;
+  int32_t dtype; /* FtDtype of every tensor */
+} FtLinBlockArgs;
+
+/* 0 if the arguments are not supported (ft_last_error() says why). */
+size_t ft_linattn_block_workspace_bytes(const FtLinBlockArgs* b, int kind);
+
+/* hipBLASLt is opened on first use (FT_EUNSUPPORTED if it cannot be found); its handle and the GEMM plans
+ * are cached per device and shape, and calls of this entry point serialise on one mutex. */
+int ft_linattn_block_fwd(const FtLinBlockArgs* b, int kind, int normalize_q, void* workspace, size_t workspace_bytes,
+                         void* stream);
 
 /* Heavy hitters: indices of the k largest entries of each row of score [rows, S] fp32, in descending
  * score order (ties: lower index first), written as int64 [rows, k].  Not in the reference, whose H2O

@@ -13,6 +13,7 @@ listed in `oracle/cases.py`'s header and exercised by `tests/test_oracle_*.py`.
 from .cases import (  # noqa: F401
     attn_forward, h2o_forward, keyformer_forward, roco_forward, ea_forward, sima_forward,
     snapkv_forward, corm_forward, corm_mask_rule, corm_margin, gemma2_forward, attn2d_forward, attn_h2o2d_forward,
+    ea_block_forward, sima_block_forward, prepare_block_inputs,
     prepare_inputs, prepare_exp_rand, heavy_hitters, roco_mean_var, chunked_over_heads,
 )
 from .noise import seeded_exp_rand, noise_u32, lowbias32  # noqa: F401

@@ -28,6 +28,9 @@ How each function is pinned (tests/test_oracle_pins.py, tests/test_oracle_golden
   attn2d_forward,    Hkv == H -> attn_forward / h2o_forward on the [1,S,H,D] views, bit-exact; Hkv < H ->
   attn_h2o2d_forward the same functions on k/v heads repeated with repeat_interleave, scores averaged per group;
                      fp64 brute force with explicit h // group indexing; unmasked rows sum to Sq.
+  ea_block_forward,  stacked identity weights, zero biases -> the core on (x, x, x), bit-exact; x == 0 -> q, k, v
+  sima_block_forward are the bias rows, V constant over tokens -> y == w_out b_v + b_out (EA); fp64 brute force with
+                     explicit loops over a non-symmetric weight (a transposed operand or a wrong split order fails).
 The reference holds no golden vectors or tests for this path, so none can be checked against; no
 function of this file is "parity unpinned".
 """
@@ -214,6 +217,48 @@ def sima_forward(q, k, v, normalize_q=True, out_dtype=None):
   kv = torch.matmul(kh.transpose(-2, -1), vf)
   out = torch.matmul(qh, kv)
   return out.transpose(1, 2).contiguous().to(out_dtype or q.dtype)
+
+
+def _linear16(x, w, b):
+  """A Linear as the .mlir writes it (transpose, dot, add: bench/ea.mlir:3-5 and :20-22), evaluated in fp32
+  from 16-bit operands and rounded once to the operand dtype: the rounding points of a 16-bit GEMM with
+  fp32 accumulation and a fused bias."""
+  y = torch.matmul(x.float(), w.float().transpose(0, 1))
+  if b is not None:
+    y = y + b.float()
+  return y.to(x.dtype)
+
+
+def _block(core, x, w_qkv, b_qkv, w_out, b_out, head_num, **kw):
+  B, S, C = x.shape
+  qkv = _linear16(x, w_qkv, b_qkv)                                          # ea.mlir:3-5
+  q, k, v = (t.reshape(B, S, head_num, C // head_num) for t in qkv.split(C, dim=2))  # :6-9 (core transposes, :10-12)
+  o = core(q, k, v, **kw)                                                   # :13-19
+  return _linear16(o.reshape(B, S, C), w_out, b_out)                        # :20-22
+
+
+def ea_block_forward(x, w_qkv, b_qkv, w_out, b_out, head_num):
+  """The whole function of bench/ea.mlir:2-23 on 16-bit tensors (the graph itself is f32; q/k/v, the core's
+  result and y are the 16-bit tensors between the stages)."""
+  return _block(ea_forward, x, w_qkv, b_qkv, w_out, b_out, head_num)
+
+
+def sima_block_forward(x, w_qkv, b_qkv, w_out, b_out, head_num, normalize_q=True):
+  """The whole function of bench/sima.mlir:2-23."""
+  return _block(sima_forward, x, w_qkv, b_qkv, w_out, b_out, head_num, normalize_q=normalize_q)
+
+
+def prepare_block_inputs(B, S, H, D, seed=0, dtype=torch.float16):
+  """x ~ N(0,1); weights ~ N(0,1/C) so that q, k, v come out ~ N(0,1) as in the core's own recipe; biases 0.1 N(0,1)."""
+  g = torch.Generator(device="cpu")
+  g.manual_seed(seed)
+  C = H * D
+  x = torch.randn(B, S, C, dtype=dtype, generator=g)
+  w_qkv = (torch.randn(3 * C, C, generator=g) / C ** 0.5).to(dtype)
+  b_qkv = (0.1 * torch.randn(3 * C, generator=g)).to(dtype)
+  w_out = (torch.randn(C, C, generator=g) / C ** 0.5).to(dtype)
+  b_out = (0.1 * torch.randn(C, generator=g)).to(dtype)
+  return x, w_qkv, b_qkv, w_out, b_out
 
 
 # ---------------------------------------------------------------------------------------------------

@@ -62,6 +62,28 @@ def sima(q, k, v, normalize_q=True):
   return O
 
 
+def linear_block(core, x, w_qkv, b_qkv, w_out, b_out, H, **kw):
+  """y[b,s,m] = sum_c core(q,k,v)[b,s,c] w_out[m,c] + b_out[m] with qkv[b,s,n] = sum_c x[b,s,c] w_qkv[n,c] + b_qkv[n],
+  q/k/v = columns [0,C) / [C,2C) / [2C,3C) of qkv, head h = channels [h D, (h+1) D).  fp64, no intermediate
+  rounding; index form (einsum subscripts), independent of the oracle's matmul / split / reshape calls."""
+  import torch
+  x64, wq, bq, wo, bo = (t.numpy().astype(np.float64) for t in (x, w_qkv, b_qkv, w_out, b_out))
+  B, S, C = x64.shape
+  D = C // H
+  qkv = np.einsum("bsc,nc->bsn", x64, wq) + bq[None, None, :]
+  parts = []
+  for i in range(3):
+    t = np.zeros((B, S, H, D))
+    for h in range(H):
+      t[:, :, h, :] = qkv[:, :, i * C + h * D:i * C + (h + 1) * D]
+    parts.append(torch.from_numpy(t))
+  o = core(*parts, **kw)            # the fp64 brute-force cores above take any float tensors
+  flat = np.zeros((B, S, C))
+  for h in range(H):
+    flat[:, :, h * D:(h + 1) * D] = o[:, :, h, :]
+  return np.einsum("bsc,mc->bsm", flat, wo) + bo[None, None, :]
+
+
 def avg_pool_same(x, kernel):
   """Stride-1 window mean over the last axis with kernel // 2 zeros on both sides, divisor = kernel."""
   x = np.asarray(x, dtype=np.float64)

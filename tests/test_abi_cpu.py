@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(lib):
   assert declared == sorted(_lib.EXPORTS)
   for name in declared:
     assert getattr(lib, name) is not None
-  assert lib.ft_abi_version() == 2 == _lib.ABI_VERSION
+  assert lib.ft_abi_version() == 3 == _lib.ABI_VERSION
 
 
 def _args(**over):
@@ -127,6 +127,24 @@ def test_linattn_and_topk_argument_checks(lib):
   assert lib.ft_topk(0x1000, 1, 16384, 9, 0x2000, None) == _lib.FT_EUNSUPPORTED
 
 
+def test_linear_block_argument_checks(lib):
+  b = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
+  need = lib.ft_linattn_block_workspace_bytes(ctypes.byref(b), _lib.FT_OP_EA)
+  C = 4 * 64
+  assert need >= 2 * 100 * 4 * C * 2 + (32 << 20) and need % 256 == 0
+  assert lib.ft_linattn_block_fwd(ctypes.byref(b), _lib.FT_OP_EA, 1, 0x10000, need - 1, None) == _lib.FT_EWORKSPACE
+  assert lib.ft_linattn_block_fwd(ctypes.byref(b), 9, 1, 0x10000, need, None) == _lib.FT_EINVAL
+  assert lib.ft_linattn_block_fwd(None, _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
+  bad = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 32, _lib.FT_F16)
+  assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(bad), _lib.FT_OP_EA) == 0
+  assert "head_dim" in lib.ft_last_error().decode()
+  assert lib.ft_linattn_block_fwd(ctypes.byref(bad), _lib.FT_OP_SIMA, 1, 0x10000, need, None) == _lib.FT_EUNSUPPORTED
+  odd = _lib.FtLinBlockArgs(0x1008, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
+  assert lib.ft_linattn_block_fwd(ctypes.byref(odd), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
+  nul = _lib.FtLinBlockArgs(0x1000, None, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
+  assert lib.ft_linattn_block_fwd(ctypes.byref(nul), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
+
+
 def test_host_noise_twin_matches_oracle_stream(lib):
   import oracle
   E = ft.ops.seeded_exp_rand(2, 3, 17, 33, 987654321987, "cpu")
@@ -145,7 +163,10 @@ def test_operator_layer_validates_like_the_reference_backend():
   f = ft.HipBuilder("h2o").build_callable()
   with pytest.raises(RuntimeError, match="arg 0 need shape"):
     f(torch.zeros(1, 8, 2, 64, dtype=torch.float16), q, q)
-  assert sorted(ft.CASES) == ["attn", "corm", "ea", "gemma2", "h2o", "kf", "roco", "sima", "snapkv"]
+  assert sorted(ft.CASES) == ["attn", "corm", "ea", "ea_block", "gemma2", "h2o", "kf", "roco", "sima", "sima_block", "snapkv"]
+  g = ft.HipBuilder("ea_block", head_num=2).build_callable()
+  with pytest.raises(RuntimeError, match="arg 0 need shape"):
+    g(torch.zeros(1, 8, 64, dtype=torch.float16), None, None, None, None)
   assert ft.get_model("snapkv").kernel_size == 5 and ft.get_model("gemma2").logit_softcapping == 50.0
   assert ft.get_model("kf").tau == 1.5 and ft.get_model("h2o").prepare.__doc__
 

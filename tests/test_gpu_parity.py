@@ -293,6 +293,63 @@ def test_ea_sima_properties(gpu):
   assert torch.allclose(a, b, rtol=1e-4, atol=1e-9)
 
 
+# ------------------------------------------------------------------ the whole .mlir block: projections around the core
+
+def block_inputs(gpu, *a, **kw):
+  host = oracle.prepare_block_inputs(*a, **kw)
+  return host, tuple(t.to(gpu) for t in host)
+
+
+@pytest.mark.parametrize("B,S,H,seed", [(2, 200, 2, 0), (1, 333, 4, 1), (1, 1, 1, 2), (3, 1024, 2, 3)])
+def test_linear_block_small(gpu, B, S, H, seed):
+  host, dev = block_inputs(gpu, B, S, H, 64, seed=seed)
+  check_o(ops.ea_block(*dev, H), oracle.ea_block_forward(*host, H))
+  # raw Q as the .mlir writes it (bench/sima.mlir:17): results of ordinary magnitude
+  check_o(ops.sima_block(*dev, H, normalize_q=False), oracle.sima_block_forward(*host, H, normalize_q=False))
+  # both sides normalised: the core's result sits in fp16's subnormal range and y ~ b_out; same rounding points
+  check_o(ops.sima_block(*dev, H), oracle.sima_block_forward(*host, H))
+  # without biases
+  x, wq, _, wo, _ = dev
+  hx, hwq, _, hwo, _ = host
+  check_o(ops.ea_block(x, wq, None, wo, None, H), oracle.ea_block_forward(hx, hwq, None, hwo, None, H))
+
+
+def test_linear_block_properties(gpu):
+  H, C = 2, 128
+  host, dev = block_inputs(gpu, 2, 256, H, 64, seed=4)
+  x, wq, bq, wo, bo = dev
+  # stacked identities and zero biases: the block is the core on (x, x, x)
+  eye = torch.eye(C, dtype=torch.float16, device=gpu)
+  z3, z1 = torch.zeros(3 * C, dtype=torch.float16, device=gpu), torch.zeros(C, dtype=torch.float16, device=gpu)
+  x4 = x.reshape(2, 256, H, 64)
+  assert torch.equal(ops.ea_block(x, torch.cat([eye, eye, eye]), z3, eye, z1, H), ops.ea(x4, x4, x4).reshape(2, 256, C))
+  # x = 0: V is its bias row for every token and passes through EA unchanged: y = w_out b_v + b_out
+  y0 = ops.ea_block(torch.zeros_like(x), wq, bq, wo, bo, H).float().cpu()
+  want = host[3].float() @ host[2][2 * C:].float() + host[4].float()
+  assert (y0 - want).abs().max().item() < 3e-3
+  # a second call with another shape and then the first again: cached plans are per shape
+  y1 = ops.ea_block(x, wq, bq, wo, bo, H)
+  ops.ea_block(x[:1, :100].contiguous(), wq, bq, wo, bo, H)
+  assert torch.equal(ops.ea_block(x, wq, bq, wo, bo, H), y1)
+  with pytest.raises(ValueError, match="weights need"):
+    ops.ea_block(x, wq[:C], bq, wo, bo, H)
+  with pytest.raises(RuntimeError, match="head_dim"):
+    ops.ea_block(x, wq, bq, wo, bo, 4)
+
+
+def test_linear_block_config5_shape(gpu):
+  """B=8 S=8192 H=16 D=64 (C = 1024) on the GPU; the oracle on 2 of the 8 batches (batches are independent)."""
+  B, S, H = 8, 8192, 16
+  host, dev = block_inputs(gpu, B, S, H, 64, seed=0)
+  y = ops.ea_block(*dev, H)
+  ys = ops.sima_block(*dev, H, normalize_q=False)
+  assert torch.isfinite(y).all() and torch.isfinite(ys).all()
+  for b in (0, 5):
+    hb = (host[0][b:b + 1],) + host[1:]
+    check_o(y[b:b + 1], oracle.ea_block_forward(*hb, H))
+    check_o(ys[b:b + 1], oracle.sima_block_forward(*hb, H, normalize_q=False))
+
+
 # ------------------------------------------------------------------ SnapKV, CoRM, Gemma2 (the other cases of the zoo)
 
 NEXT_SMALL = [(1, 128, 2, 128, 0), (2, 200, 3, 128, 2), (1, 333, 2, 64, 5), (1, 1, 2, 64, 4), (1, 700, 2, 128, 7)]

@@ -161,6 +161,31 @@ def test_sima_invariants_and_brute_force():
   assert torch.allclose(got, want, rtol=1e-4, atol=1e-8)
 
 
+def test_linear_block_identity_bias_and_brute_force():
+  B, S, H, D = 2, 24, 2, 64
+  C = H * D
+  x, w_qkv, b_qkv, w_out, b_out = oracle.prepare_block_inputs(B, S, H, D, seed=8)
+  # fp64 index-form brute force; a transposed weight, a swapped q/k/v slot or a wrong head split fails it
+  for fn, core, kw in ((oracle.ea_block_forward, brute.ea, {}), (oracle.sima_block_forward, brute.sima, {}),
+                       (oracle.sima_block_forward, brute.sima, {"normalize_q": False})):
+    got = fn(x, w_qkv, b_qkv, w_out, b_out, H, **kw).float().numpy()
+    ref = brute.linear_block(core, x, w_qkv, b_qkv, w_out, b_out, H, **kw)
+    assert np.abs(got - ref).max() <= 4e-3 * max(1.0, np.abs(ref).max()), (fn.__name__, kw)
+  # stacked identities and zero biases: the block is the core on (x, x, x), bit for bit
+  eye = torch.eye(C, dtype=torch.float16)
+  z3, z1 = torch.zeros(3 * C, dtype=torch.float16), torch.zeros(C, dtype=torch.float16)
+  x4 = x.reshape(B, S, H, D)
+  assert torch.equal(oracle.ea_block_forward(x, torch.cat([eye, eye, eye]), z3, eye, z1, H),
+                     oracle.ea_forward(x4, x4, x4).reshape(B, S, C))
+  assert torch.equal(oracle.sima_block_forward(x, torch.cat([eye, eye, eye]), z3, eye, z1, H),
+                     oracle.sima_forward(x4, x4, x4).reshape(B, S, C))
+  # x = 0: q, k, v are their bias rows for every token; V constant over tokens passes through EA unchanged,
+  # so y = w_out b_v + b_out (b_v = the third slot of the fused bias)
+  y0 = oracle.ea_block_forward(torch.zeros_like(x), w_qkv, b_qkv, w_out, b_out, H).float()
+  want = w_out.float() @ b_qkv[2 * C:].float() + b_out.float()
+  assert (y0 - want).abs().max() < 2e-3
+
+
 # ------------------------------------------------------------------ epilogues, recipes, chunking
 
 def test_heavy_hitters_and_gap_rule():
