@@ -106,11 +106,17 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   auto stage_q = [&](int t, char* dst) {
     if (t < ntiles) stQ.issue(i_begin + t * BQ, min(BQ, p.Sq - (i_begin + t * BQ)), dst);
   };
-  // rows of tile t: negated normaliser (-inf past Sq, so that those rows contribute exp2(-inf) = 0) and noise row term
-  auto stage_rows = [&](int t) {
+  // rows of tile t: negated normaliser (-inf past Sq, so that those rows contribute exp2(-inf) = 0) and noise
+  // row term.  The normaliser is fetched one iteration before it is parked in LDS, so that no wave sits
+  // out a global-memory round trip inside the loop.
+  auto load_rows = [&](int t) -> float {
+    const int i = i_begin + t * BQ + threadIdx.x;
+    return (t < ntiles && threadIdx.x < BQ && i < p.Sq) ? lse_bh[i] : POS_INF;
+  };
+  auto store_rows = [&](int t, float lse_i) {
     if (t < ntiles && threadIdx.x < BQ) {
       const int i = i_begin + t * BQ + threadIdx.x;
-      float nl = i < p.Sq ? -lse_bh[i] : NEG_INF;  // negated: one fma per logit
+      float nl = -lse_i;  // negated: one fma per logit
       // CoRM rule: p_ij >= 1 / (i + 1)  <=>  log2 p_ij + log2(i + 1) >= 0, so no exponential is needed
       if (MODE == kStatCormRule) nl += __builtin_amdgcn_logf((float)(i + 1));
       ldsLse[(t & 1) * BQ + threadIdx.x] = nl;
@@ -251,7 +257,8 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
     // ---- prologue: Q[0], Q[1] in flight; rows of tile 0; scores of tile 0
     stage_q(0, ldsQ0);
     stage_q(1, ldsQ1);
-    stage_rows(0);
+    store_rows(0, load_rows(0));
+    float lse_next = load_rows(1);  // rows of the tile after the current one, in flight
     wait_vmem();
     __syncthreads();
     qk(S0, ldsQ0);
@@ -263,7 +270,8 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
       wait_vmem();
       __syncthreads();
       stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
-      stage_rows(t + 1);
+      store_rows(t + 1, lse_next);
+      lse_next = load_rows(t + 2);
       // every row of this tile above the diagonal for all 32 keys of the wave: nothing to add
       const bool skip = CAUSAL && (wave_key0 > i_begin + t * BQ + BQ - 1 + p.off);
       if (!skip) reduce_tile(std::true_type{}, S0, t);
@@ -274,7 +282,8 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
       wait_vmem();
       __syncthreads();
       stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
-      stage_rows(t + 1);
+      store_rows(t + 1, lse_next);
+      lse_next = load_rows(t + 2);
       reduce_tile(std::false_type{}, S0, t);
       qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
       ++t;
@@ -286,14 +295,16 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
       wait_vmem();
       __syncthreads();
       stage_q(t + 2, qa_buf);
-      stage_rows(t + 1);
+      store_rows(t + 1, lse_next);
+      lse_next = load_rows(t + 2);
       qk(S1, qb_buf);
       reduce_tile(std::false_type{}, S0, t);
       sched_tile();
       wait_vmem();
       __syncthreads();
       stage_q(t + 3, qb_buf);
-      stage_rows(t + 2);
+      store_rows(t + 2, lse_next);
+      lse_next = load_rows(t + 3);
       qk(S0, qa_buf);  // tile t + 2; past the last tile this reads stale LDS and is discarded
       reduce_tile(std::false_type{}, S1, t + 1);
       sched_tile();
