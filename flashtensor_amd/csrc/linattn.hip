@@ -52,14 +52,23 @@ struct LinParams {
   uint16_t* w;      // [BH][2][64 e][64 d] fp16: hi, lo * 2^11
   float* winv;      // [BH][4] 1 / scale of each block of 16 output channels
   int B, H, S;
-  int nch;              // chunks per (b, h)
-  int tiles_per_chunk;  // 128-token tiles per chunk
+  int nch;              // chunks per (b, h) of the K/V pass
+  int tiles_per_chunk;  // 128-token tiles per chunk of the K/V pass
+  int out_nch;              // the same for the output pass (its chunks are independent of the K/V pass's)
+  int out_tiles_per_chunk;
 };
 
-static void lin_plan(const FtAttnArgs& a, int* nch, int* tpc) {
+// Splits the sequence of every (b, h) into chunks so that about `workgroups` workgroups exist.  The K/V pass
+// keeps two workgroups per CU and pays a pipeline fill, a four-wave fold and a partial-result write per
+// workgroup, so it wants one round of them (512); the output pass runs more workgroups per CU and has no
+// epilogue, so more, shorter ones balance better (measured in one process at B8 H16 S8192, EA / SimA:
+// 1024 + 1024 workgroups 148 / 147 us, 512 + 1024 136 / 139, 512 + 2048 135 / 137, 512 + 4096 143 / 141).
+constexpr int kKvWorkgroups = 512, kOutWorkgroups = 2048;
+
+static void lin_plan(const FtAttnArgs& a, int workgroups, int* nch, int* tpc) {
   const int ntiles = (a.Sq + kLinTile - 1) / kLinTile;
   const int64_t bh = (int64_t)a.B * a.H;
-  int want = (int)((1024 + bh - 1) / bh);  // aim for >= ~1024 workgroups
+  int want = (int)((workgroups + bh - 1) / bh);
   if (want < 1) want = 1;
   int t = (ntiles + want - 1) / want;
   if (t < 1) t = 1;
@@ -70,7 +79,7 @@ static void lin_plan(const FtAttnArgs& a, int* nch, int* tpc) {
 
 size_t linattn_workspace_bytes(const FtAttnArgs& a, int) {
   int nch, tpc;
-  lin_plan(a, &nch, &tpc);
+  lin_plan(a, kKvWorkgroups, &nch, &tpc);
   const size_t bh = (size_t)a.B * a.H;
   size_t bytes = bh * nch * kPartStride * sizeof(float);
   bytes += bh * 2 * kLinD * kLinD * sizeof(uint16_t);
@@ -567,8 +576,8 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   char* ost = otr + wave * SUB * OROW;
   char* tq = s_q[wave];
 
-  const int tok_begin = ch * p.tiles_per_chunk * kLinTile;
-  const int tok_end = min(p.S, tok_begin + p.tiles_per_chunk * kLinTile);
+  const int tok_begin = ch * p.out_tiles_per_chunk * kLinTile;
+  const int tok_end = min(p.S, tok_begin + p.out_tiles_per_chunk * kLinTile);
   const int nsub = (tok_end - tok_begin + SUB - 1) / SUB;
   const int nmine = nsub > wave ? (nsub - wave + kLinWaves - 1) / kLinWaves : 0;
 
@@ -723,7 +732,8 @@ hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int ou
   p.B = a.B;
   p.H = a.H;
   p.S = a.Sq;
-  lin_plan(a, &p.nch, &p.tiles_per_chunk);
+  lin_plan(a, kKvWorkgroups, &p.nch, &p.tiles_per_chunk);
+  lin_plan(a, kOutWorkgroups, &p.out_nch, &p.out_tiles_per_chunk);
   const bool ea = kind == FT_OP_EA;
   const bool nq = !ea && normalize_q;
   const bool f32 = out_dtype == FT_F32;
@@ -735,7 +745,7 @@ hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int ou
   base += bh * 2 * kLinD * kLinD * sizeof(uint16_t);
   p.winv = reinterpret_cast<float*>(base);
 
-  const dim3 grid1((unsigned)(bh * p.nch)), blk(kLinThreads);
+  const dim3 grid1((unsigned)(bh * p.nch)), grid3((unsigned)(bh * p.out_nch)), blk(kLinThreads);
   if (ea)
     hipLaunchKernelGGL((linattn_kv_kernel<true, false>), grid1, blk, 0, s, p);
   else if (nq)
@@ -753,14 +763,14 @@ hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int ou
   if (e != hipSuccess) return e;
   if (ea) {
     if (f32)
-      hipLaunchKernelGGL((linattn_out_kernel<true, true>), grid1, blk, 0, s, p);
+      hipLaunchKernelGGL((linattn_out_kernel<true, true>), grid3, blk, 0, s, p);
     else
-      hipLaunchKernelGGL((linattn_out_kernel<true, false>), grid1, blk, 0, s, p);
+      hipLaunchKernelGGL((linattn_out_kernel<true, false>), grid3, blk, 0, s, p);
   } else {
     if (f32)
-      hipLaunchKernelGGL((linattn_out_kernel<false, true>), grid1, blk, 0, s, p);
+      hipLaunchKernelGGL((linattn_out_kernel<false, true>), grid3, blk, 0, s, p);
     else
-      hipLaunchKernelGGL((linattn_out_kernel<false, false>), grid1, blk, 0, s, p);
+      hipLaunchKernelGGL((linattn_out_kernel<false, false>), grid3, blk, 0, s, p);
   }
   return hipGetLastError();
 }
