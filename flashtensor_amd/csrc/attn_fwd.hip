@@ -208,7 +208,8 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       const int jl = 32 * mbk + 8 * (r >> 2) + (r & 3);
       return jl > lim ? NEG_INF : s[mbk][r];
     };
-    // four independent chains, then a short tree: the reduction is latency-, not throughput-bound
+    // four independent chains, then a short tree: the reduction is latency-, not throughput-bound.  Only
+    // three-operand maxima: a two-operand fmaxf on MFMA results costs two extra NaN-quieting moves.
     float m4[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -216,10 +217,11 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
       m4[c] = max3(at(mbk, r0), at(mbk, r0 + 1), at(mbk, r0 + 2));
       m4[c] = max3(m4[c], at(mbk, r0 + 3), at(mbk, r0 + 4));
       m4[c] = max3(m4[c], at(mbk, r0 + 5), at(mbk, r0 + 6));
-      m4[c] = __builtin_fmaxf(m4[c], at(mbk, r0 + 7));
     }
-    float amax = __builtin_fmaxf(max3(m4[0], m4[1], m4[2]), m4[3]);
-    amax = __builtin_fmaxf(amax, xchg32(amax));
+    const float t0 = max3(m4[0], at(0, 7), at(0, 15)), t1 = max3(m4[1], at(1, 7), at(1, 15));
+    float amax = max3(max3(t0, t1, m4[2]), m4[3], m4[3]);
+    const float other = xchg32(amax);
+    amax = max3(amax, other, other);
     if (EMU)
       rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
     else
