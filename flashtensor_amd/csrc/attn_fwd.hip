@@ -6,7 +6,9 @@
 // column-statistics pass consumes, and in the KeyFormer modes the normaliser of the Gumbel-perturbed
 // softmax of kf.py:36-39 instead.
 //
-// Mapping.  One workgroup = 128 query rows of one (b, h), 4 waves x 32 rows; keys are streamed in tiles
+// Mapping.  One workgroup = 32 WAVES query rows of one (b, h), one wave per 32 rows (4 waves and two
+// workgroups per CU, or 8 waves and one: the same two waves per SIMD, but a staged K/V tile then serves
+// twice as many rows); keys are streamed in tiles
 // of 64 through double-buffered LDS (direct global->LDS loads).  Each wave computes the TRANSPOSED score
 // block S^T = K Q^T with v_mfma_f32_32x32x16: a lane then owns one query (column l % 32) and 16 of the
 // 32 keys of each block, so the online-softmax row max / row sum are in-lane reductions plus a single
@@ -20,9 +22,7 @@
 
 namespace ft {
 
-constexpr int kAttnBM = 128;
 constexpr int kAttnBN = 64;
-constexpr int kAttnThreads = 256;
 
 // Rescale threshold of the running maximum in log2 units: the stale maximum is kept (and O, l are not
 // rescaled) while the new row maximum exceeds it by less than this, so unnormalised probabilities stay
@@ -31,9 +31,9 @@ constexpr float kRescaleSlack = 6.f;
 
 enum TileMode { kTileFast = 0, kTileMasked = 1, kTileIdle = 2 };
 
-template <typename T, int D, bool CAUSAL, bool EMU, int KF>
-__global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKernelParams p) {
-  constexpr int BM = kAttnBM, BN = kAttnBN, NT = kAttnThreads;
+template <typename T, int D, bool CAUSAL, bool EMU, int KF, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const AttnKernelParams p) {
+  constexpr int BM = 32 * WAVES, BN = kAttnBN, NT = 64 * WAVES;
   constexpr int KSTEPS = D / 16;
   constexpr int DB = D / 32;
   typedef TileGeom<D> G;
@@ -546,11 +546,32 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnKer
 // ---------------------------------------------------------------------------------------------------
 // host-side launcher
 
+static int device_cu_count() {
+  static int cus[16] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    cus[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cus[dev];
+}
+
 template <typename T, int D, bool CAUSAL, bool EMU, int KF>
 static hipError_t launch_one(const AttnKernelParams& p, hipStream_t stream) {
-  const int nMB = (p.Sq + kAttnBM - 1) / kAttnBM;
+  // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
+  // there are half as many of them: used on the pipelined fp16 paths once they still fill the chip twice
+  constexpr bool kHas8 = std::is_same<T, F16>::value && (KF == kKfNone || KF == kKfSeededTau1 || KF == kKfSeededFast);
+  if constexpr (kHas8) {
+    const int64_t n8 = (int64_t)((p.Sq + 255) / 256) * p.B * p.H;
+    if (n8 >= 2 * (int64_t)device_cu_count()) {
+      hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 8>), dim3((unsigned)n8), dim3(512), 0, stream, p);
+      return hipGetLastError();
+    }
+  }
+  const int nMB = (p.Sq + 127) / 128;
   dim3 grid((unsigned)(nMB * p.B * p.H));
-  hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF>), grid, dim3(kAttnThreads), 0, stream, p);
+  hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 4>), grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 
