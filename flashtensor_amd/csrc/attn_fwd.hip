@@ -42,9 +42,9 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   constexpr bool kIsF16 = __is_same(typename T::elem, _Float16);
   constexpr bool kKfFast = KF == kKfSeededTau1 || KF == kKfSeededFast;           // seeded noise inside the packed path
   constexpr bool kSeeded = KF == kKfSeeded || kKfFast;
-  // variants served by the pipelined fast path: fp16 plain softmax with either treatment of the logits, and
-  // the packed seeded KeyFormer modes
-  constexpr bool kFastMasked = kIsF16 && ((EMU && kKfFast) || KF == kKfNone);
+  // variants served by the pipelined fast path: the plain softmax in either type with either treatment of the
+  // logits, and the packed seeded KeyFormer modes (fp16)
+  constexpr bool kFastMasked = (kIsF16 && EMU && kKfFast) || KF == kKfNone;
   static_assert(!kKfFast || (kIsF16 && EMU), "the packed KeyFormer modes exist for fp16 with reference rounding only");
   // Software pipeline across tiles: the QK^T MFMAs of tile it+1 are issued in the same iteration as the
   // softmax (VALU) and PV MFMAs of tile it, so the matrix and vector pipes overlap inside one wave.
@@ -223,7 +223,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     const float other = xchg32(amax);
     amax = max3(amax, other, other);
     if (EMU)
-      rescale((float)(_Float16)((float)(_Float16)amax * p.logit_mul) * kLog2e);
+      rescale(T::to_float(T::from_float(T::to_float(T::from_float(amax)) * p.logit_mul)) * kLog2e);
     else
       rescale(amax * p.logit_mul);  // logit_mul = log2e / sqrt(D) when the logits stay in fp32
   };
@@ -231,7 +231,6 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0, int buf) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const float neg_m = -m_run;
-    const half2v ones = {(_Float16)1.f, (_Float16)1.f};
     const half2v pk_hi = __builtin_bit_cast(half2v, p.pk_hi2), pk_lo = __builtin_bit_cast(half2v, p.pk_lo2);
     // local key index of register r is 32 mbk + 8 (r / 4) + 4 g + r % 4; it is visible iff <= lim + 4 g
     const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0 - 4 * g;
@@ -241,9 +240,9 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 #pragma unroll
     for (int blk = 0; blk < 4; ++blk) {
       const int mbk = blk >> 1, rb = (blk & 1) * 8;
-      half2v t2[4];
       float x[8];
-      if constexpr (EMU) {
+      if constexpr (EMU && kIsF16) {
+        half2v t2[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float2v a2 = {s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]};
@@ -251,12 +250,25 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
           // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
           t2[i] = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
         }
-      }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        x[i] = EMU ? __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m)
-                   : __builtin_fmaf(s[mbk][rb + i], p.logit_mul, neg_m);
-        if (MASKED) {
+        for (int i = 0; i < 8; ++i) x[i] = __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m);
+      } else if constexpr (EMU) {
+        // bf16: round QK^T, multiply by the tuned constant (== dividing by sqrt(D) in bf16), round again; the
+        // conversions handle two elements each, unpacking a half is a shift or a mask
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t h2 = T::pack2(s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]);
+          const uint32_t t2 = T::pack2(T::lo(h2) * p.logit_mul, T::hi(h2) * p.logit_mul);
+          x[2 * i] = __builtin_fmaf(T::lo(t2), kLog2e, neg_m);
+          x[2 * i + 1] = __builtin_fmaf(T::hi(t2), kLog2e, neg_m);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = __builtin_fmaf(s[mbk][rb + i], p.logit_mul, neg_m);
+      }
+      if (MASKED) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
           const int jl = 32 * mbk + 8 * ((rb + i) >> 2) + ((rb + i) & 3);
           x[i] = (jl > lim) ? NEG_INF : x[i];
         }
@@ -284,10 +296,8 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float2v p2 = {x[2 * i], x[2 * i + 1]};
-        const half2v ph = __builtin_convertvector(p2, half2v);
-        l_run = __builtin_amdgcn_fdot2(ph, ones, l_run, false);  // row sum of the fp16 P the MFMA consumes
-        pw[blk][i] = __builtin_bit_cast(uint32_t, ph);           // whole 32-bit words: no 16-bit shuffles
+        pw[blk][i] = T::pack2(x[2 * i], x[2 * i + 1]);  // whole 32-bit words: no 16-bit shuffles
+        l_run = T::add2(pw[blk][i], l_run);             // row sum of the 16-bit P the MFMA consumes
       }
     }
 #pragma unroll
@@ -561,7 +571,7 @@ template <typename T, int D, bool CAUSAL, bool EMU, int KF>
 static hipError_t launch_one(const AttnKernelParams& p, hipStream_t stream) {
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
   // there are half as many of them: used on the pipelined fp16 paths once they still fill the chip twice
-  constexpr bool kHas8 = std::is_same<T, F16>::value && (KF == kKfNone || KF == kKfSeededTau1 || KF == kKfSeededFast);
+  constexpr bool kHas8 = KF == kKfNone || KF == kKfSeededTau1 || KF == kKfSeededFast;
   if constexpr (kHas8) {
     const int64_t n8 = (int64_t)((p.Sq + 255) / 256) * p.B * p.H;
     if (n8 >= 2 * (int64_t)device_cu_count()) {

@@ -26,10 +26,10 @@ constexpr int kColBQ = 64;   // query rows per tile
 constexpr int kColThreads = 256;
 
 // waves per SIMD the register budget is sized for: the sum / sum-of-squares variants with a short logit chain
-// (packed fp16 rounding, or logits kept in fp32) fit three
+// (packed rounding, or logits kept in fp32) fit three
 template <typename T, bool EMU, int MODE>
 constexpr int colstats_waves_per_simd() {
-  return ((__is_same(typename T::elem, _Float16) || !EMU) && (MODE == kStatSum || MODE == kStatSumSq)) ? 3 : 2;
+  return (MODE == kStatSum || MODE == kStatSumSq) ? 3 : 2;
 }
 
 template <typename T, int D, bool CAUSAL, bool EMU, int MODE>
@@ -179,6 +179,15 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
         if (kPlainF32 && !KFM && !KFP) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) x[e] = __builtin_fmaf(s[mbk][4 * q4 + e], p.logit_mul, nlse4[e]);
+        } else if (EMU && !kPacked && !KFM && !KFP) {
+          // bf16: round QK^T, multiply by the tuned constant (== dividing by sqrt(D) in bf16), round again
+#pragma unroll
+          for (int e = 0; e < 4; e += 2) {
+            const uint32_t h2 = T::pack2(s[mbk][4 * q4 + e], s[mbk][4 * q4 + e + 1]);
+            const uint32_t t2 = T::pack2(T::lo(h2) * p.logit_mul, T::hi(h2) * p.logit_mul);
+            x[e] = __builtin_fmaf(T::lo(t2), kLog2e, nlse4[e]);
+            x[e + 1] = __builtin_fmaf(T::hi(t2), kLog2e, nlse4[e + 1]);
+          }
         } else if (kPacked && !KFM) {
 #pragma unroll
           for (int e = 0; e < 4; e += 2) {

@@ -15,6 +15,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
@@ -40,6 +41,17 @@ struct F16 {
     return __builtin_bit_cast(uint16_t, h);
   }
   static __device__ __forceinline__ float to_float(uint16_t x) { return (float)__builtin_bit_cast(_Float16, x); }
+  // two floats rounded to the storage type in one 32-bit word; its halves as floats; acc + lo + hi
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const float2v v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2v));
+  }
+  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(half2v, w)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(half2v, w)[1]; }
+  static __device__ __forceinline__ float add2(uint32_t w, float acc) {
+    const half2v ones = {(_Float16)1.f, (_Float16)1.f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, w), ones, acc, false);
+  }
 };
 struct BF16 {
   typedef bf16x8 vec8;
@@ -48,13 +60,20 @@ struct BF16 {
   static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ uint16_t from_float(float x) {  // round to nearest even
-    uint32_t u = __builtin_bit_cast(uint32_t, x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+  static __device__ __forceinline__ uint16_t from_float(float x) {  // round to nearest even (v_cvt_pk_bf16_f32)
+    return __builtin_bit_cast(uint16_t, (__bf16)x);
   }
   static __device__ __forceinline__ float to_float(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const float2v v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+  static __device__ __forceinline__ float add2(uint32_t w, float acc) {
+    const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
+  }
 };
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
