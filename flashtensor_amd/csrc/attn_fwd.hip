@@ -44,7 +44,8 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   constexpr bool kSeeded = KF == kKfSeeded || kKfFast;
   // variants served by the pipelined fast path: the plain softmax in either type with either treatment of the
   // logits, and the packed seeded KeyFormer modes (fp16)
-  constexpr bool kFastMasked = (kIsF16 && EMU && kKfFast) || KF == kKfNone;
+  constexpr bool kFastMasked = (kIsF16 && EMU && kKfFast) || KF == kKfNone || KF == kKfSoftcap;
+  constexpr bool kCap = KF == kKfSoftcap;
   static_assert(!kKfFast || (kIsF16 && EMU), "the packed KeyFormer modes exist for fp16 with reference rounding only");
   // Software pipeline across tiles: the QK^T MFMAs of tile it+1 are issued in the same iteration as the
   // softmax (VALU) and PV MFMAs of tile it, so the matrix and vector pipes overlap inside one wave.
@@ -200,6 +201,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // MASKED (tiles that straddle the diagonal or the end of K): hidden keys are left out of the maximum, so
   // that a row whose largest visible logit defines the stabiliser gets exp2(0) = 1 for it exactly (row 0
   // of a causal problem then has the normaliser of the reference, bit for bit).
+  const float rcp_cap = kCap ? 1.f / p.softcap : 0.f;
   auto fast_max = [&](auto masked_tag, const float16v (&s)[2], int n0) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0 - 4 * g;
@@ -222,10 +224,18 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     float amax = max3(max3(t0, t1, m4[2]), m4[3], m4[3]);
     const float other = xchg32(amax);
     amax = max3(amax, other, other);
-    if (EMU)
-      rescale(T::to_float(T::from_float(T::to_float(T::from_float(amax)) * p.logit_mul)) * kLog2e);
-    else
+    // soft-cap: the cap is monotonic as well (a product with a positive constant, tanh, roundings), so the
+    // maximum of the capped logits is the capped maximum
+    auto r16 = [](float x) { return T::to_float(T::from_float(x)); };
+    if (EMU) {
+      float t = r16(r16(amax) * p.logit_mul);
+      if (kCap) t = r16(r16(tanh_exp_form(r16(t * rcp_cap))) * p.softcap);
+      rescale(t * kLog2e);
+    } else if (kCap) {
+      rescale(p.softcap * tanh_exp_form(amax * (p.logit_mul * (1.f / kLog2e)) * rcp_cap) * kLog2e);
+    } else {
       rescale(amax * p.logit_mul);  // logit_mul = log2e / sqrt(D) when the logits stay in fp32
+    }
   };
   // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.
   auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0, int buf) {
@@ -251,7 +261,9 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
           t2[i] = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m);
+        for (int i = 0; i < 8; ++i)
+          x[i] = kCap ? (float)t2[i >> 1][i & 1] * (rcp_cap * 0.125f)  // logit / cap, rounded below
+                      : __builtin_fmaf((float)t2[i >> 1][i & 1], kLog2e / 8.f, neg_m);
       } else if constexpr (EMU) {
         // bf16: round QK^T, multiply by the tuned constant (== dividing by sqrt(D) in bf16), round again; the
         // conversions handle two elements each, unpacking a half is a shift or a mask
@@ -259,12 +271,35 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
         for (int i = 0; i < 4; ++i) {
           const uint32_t h2 = T::pack2(s[mbk][rb + 2 * i], s[mbk][rb + 2 * i + 1]);
           const uint32_t t2 = T::pack2(T::lo(h2) * p.logit_mul, T::hi(h2) * p.logit_mul);
-          x[2 * i] = __builtin_fmaf(T::lo(t2), kLog2e, neg_m);
-          x[2 * i + 1] = __builtin_fmaf(T::hi(t2), kLog2e, neg_m);
+          x[2 * i] = kCap ? T::lo(t2) * rcp_cap : __builtin_fmaf(T::lo(t2), kLog2e, neg_m);
+          x[2 * i + 1] = kCap ? T::hi(t2) * rcp_cap : __builtin_fmaf(T::hi(t2), kLog2e, neg_m);
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = __builtin_fmaf(s[mbk][rb + i], p.logit_mul, neg_m);
+        for (int i = 0; i < 8; ++i)
+          x[i] = kCap ? s[mbk][rb + i] * (p.logit_mul * (1.f / kLog2e) * rcp_cap) : __builtin_fmaf(s[mbk][rb + i], p.logit_mul, neg_m);
+      }
+      if constexpr (kCap) {
+        // Gemma2's soft-cap, cap * tanh(logit / cap): three 16-bit tensor ops in the reference
+        // (cases/kernels/gemma2.py:31-33), each rounded when the reference's rounding is reproduced
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float y0 = x[2 * i], y1 = x[2 * i + 1];
+          if (EMU) {
+            const uint32_t w = T::pack2(y0, y1);
+            y0 = T::lo(w), y1 = T::hi(w);
+          }
+          float z0 = tanh_exp_form(y0), z1 = tanh_exp_form(y1);
+          if (EMU) {
+            const uint32_t w = T::pack2(z0, z1);
+            const uint32_t c = T::pack2(T::lo(w) * p.softcap, T::hi(w) * p.softcap);
+            x[2 * i] = __builtin_fmaf(T::lo(c), kLog2e, neg_m);
+            x[2 * i + 1] = __builtin_fmaf(T::hi(c), kLog2e, neg_m);
+          } else {
+            x[2 * i] = __builtin_fmaf(z0 * p.softcap, kLog2e, neg_m);
+            x[2 * i + 1] = __builtin_fmaf(z1 * p.softcap, kLog2e, neg_m);
+          }
+        }
       }
       if (MASKED) {
 #pragma unroll
@@ -423,7 +458,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   auto fast_tile = [&](auto masked_tag, auto stage_tag, float16v (&s_cur)[2], float16v (&s_next)[2], const char* tk_next,
                        const char* tv, int n0, int it, char* k_dst, char* v_dst) {
     constexpr bool STAGE = decltype(stage_tag)::value;
-    constexpr int kValuGroup = kKfFast ? 16 : 6;  // vector instructions placed after each MFMA
+    constexpr int kValuGroup = kKfFast ? 16 : kCap ? 14 : 6;  // vector instructions placed after each MFMA
     vec8 pb[4];
     // STAGE: the direct-to-LDS loads of K[it+2] and V[it+1] (both full tiles) are issued from inside this
     // block, one every few MFMAs.  Issued back to back they fill the texture-address queue (one 1 KB load
@@ -571,7 +606,7 @@ template <typename T, int D, bool CAUSAL, bool EMU, int KF>
 static hipError_t launch_one(const AttnKernelParams& p, hipStream_t stream) {
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
   // there are half as many of them: used on the pipelined fp16 paths once they still fill the chip twice
-  constexpr bool kHas8 = KF == kKfNone || KF == kKfSeededTau1 || KF == kKfSeededFast;
+  constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast;
   if constexpr (kHas8) {
     const int64_t n8 = (int64_t)((p.Sq + 255) / 256) * p.B * p.H;
     if (n8 >= 2 * (int64_t)device_cu_count()) {

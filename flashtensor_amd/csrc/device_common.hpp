@@ -112,6 +112,12 @@ __device__ __forceinline__ float tanh_f32(float y) {
   return a < 0.25f ? poly : big;
 }
 
+// tanh as 1 - 2 / (e^2y + 1) for either sign: absolute error ~1e-7 (cancellation for small |y|), which is
+// enough where the result is rounded to 16 bits or only shifts a logit by that much; four instructions.
+__device__ __forceinline__ float tanh_exp_form(float y) {
+  return __builtin_fmaf(-2.f, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(y * (2.f * kLog2e)) + 1.f), 1.f);
+}
+
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
 // ---------------------------------------------------------------------------------------------------
