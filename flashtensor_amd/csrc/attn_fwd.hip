@@ -315,19 +315,20 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
         const uint32_t* col = ldsCol + buf * BN + 32 * mbk + 2 * rb + 4 * g;
         const uint4v c0 = *reinterpret_cast<const uint4v*>(col), c1 = *reinterpret_cast<const uint4v*>(col + 8);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          ee[i] = -kLn2 * __builtin_amdgcn_logf(noise_uniform(a_i, i < 4 ? c0[i] : c1[i - 4]));
+        for (int i = 0; i < 8; ++i)  // log2 u = -E / ln 2 (negative): the constant factor is applied once, at the end
+          ee[i] = __builtin_amdgcn_logf(noise_uniform(a_i, i < 4 ? c0[i] : c1[i - 4]));
         if constexpr (KF == kKfSeededFast) {
+          const float shift = -kLog2Ln2 * p.inv_tau;
 #pragma unroll
           for (int i = 0; i < 8; ++i)  // exp2(((t - m) log2e - log2 E) / tau); hidden keys carry x = -inf
-            l_kf += __builtin_amdgcn_exp2f((x[i] - __builtin_amdgcn_logf(ee[i])) * p.inv_tau);
+            l_kf += __builtin_amdgcn_exp2f(__builtin_fmaf(x[i] - __builtin_amdgcn_logf(-ee[i]), p.inv_tau, shift));
         }
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) x[i] = __builtin_amdgcn_exp2f(x[i]);
       if constexpr (KF == kKfSeededTau1) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) l_kf = __builtin_fmaf(x[i], __builtin_amdgcn_rcpf(ee[i]), l_kf);  // exp(t - m) / E
+        for (int i = 0; i < 8; ++i) l_kf = __builtin_fmaf(x[i], __builtin_amdgcn_rcpf(ee[i]), l_kf);  // -ln2 exp(t - m) / E
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -582,6 +583,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   }
   if (KF == kKfTensor || kSeeded) {
     l_kf += xchg32(l_kf);
+    if (KF == kKfSeededTau1) l_kf *= -kLog2e;  // the sum was taken over 1 / log2 u = -ln2 / E
     // packed modes: the perturbed sum shares the plain softmax's stabiliser, scaled by 1 / tau
     const float base = KF == kKfSeededTau1 ? m_run : KF == kKfSeededFast ? m_run * p.inv_tau : m_kf;
     if (qi < p.Sq && g == 0) p.lse_kf[(int64_t)bh * p.Sq + qi] = base + __builtin_amdgcn_logf(l_kf);

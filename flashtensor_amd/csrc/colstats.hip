@@ -119,6 +119,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
       float nl = -lse_i;  // negated: one fma per logit
       // CoRM rule: p_ij >= 1 / (i + 1)  <=>  log2 p_ij + log2(i + 1) >= 0, so no exponential is needed
       if (MODE == kStatCormRule) nl += __builtin_amdgcn_logf((float)(i + 1));
+      if (MODE == kStatKfSeededFast) nl -= kLog2Ln2 * p.inv_tau;  // the constant part of -log2(E) / tau
       ldsLse[(t & 1) * BQ + threadIdx.x] = nl;
       if (kSeeded) ldsRow[(t & 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)i);
     }
@@ -197,8 +198,9 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
             const half2v t2 = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
             if (MODE == kStatKfSeededFast) {
               // ((t log2e - log2 E) / tau) - lse: E = -ln u in [6e-8, 16.7]
-              const float l0 = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(noise_uniform(row4[e], b_j)));
-              const float l1 = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(noise_uniform(row4[e + 1], b_j)));
+              // log2 E = log2(-log2 u) + log2(ln 2); the constant rides in the row normaliser staged in LDS
+              const float l0 = __builtin_amdgcn_logf(-__builtin_amdgcn_logf(noise_uniform(row4[e], b_j)));
+              const float l1 = __builtin_amdgcn_logf(-__builtin_amdgcn_logf(noise_uniform(row4[e + 1], b_j)));
               x[e] = __builtin_fmaf(__builtin_fmaf((float)t2[0], kLog2e / 8.f, -l0), p.inv_tau, nlse4[e]);
               x[e + 1] = __builtin_fmaf(__builtin_fmaf((float)t2[1], kLog2e / 8.f, -l1), p.inv_tau, nlse4[e + 1]);
             } else {
@@ -238,8 +240,8 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
             best[e] = fmaxf(best[e], xv);
           } else {
             float pr = __builtin_amdgcn_exp2f(xv);
-            if (MODE == kStatKfSeededTau1)  // exp(t - lse) / E
-              pr *= __builtin_amdgcn_rcpf(-kLn2 * __builtin_amdgcn_logf(noise_uniform(row4[e], b_j)));
+            if (MODE == kStatKfSeededTau1)  // exp(t - lse) / log2 u = -ln2 exp(t - lse) / E; the factor is applied to the total
+              pr *= __builtin_amdgcn_rcpf(__builtin_amdgcn_logf(noise_uniform(row4[e], b_j)));
             if (MODE == kStatCormTensor) {
               best[e] = fmaxf(best[e], pr - er[mbk][4 * q4 + e] * (1.f - kCormSlack));
             } else {
@@ -322,6 +324,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
 
   float tot = (sum[0] + sum[1]) + (sum[2] + sum[3]);
   tot += xchg32(tot);
+  if (MODE == kStatKfSeededTau1) tot *= -kLog2e;
   float totsq = (sumsq[0] + sumsq[1]) + (sumsq[2] + sumsq[3]);
   if (MODE == kStatSumSq) totsq += xchg32(totsq);
   float top = fmaxf(fmaxf(best[0], best[1]), fmaxf(best[2], best[3]));

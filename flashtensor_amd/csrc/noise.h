@@ -49,7 +49,16 @@ FT_HD uint32_t noise_col(NoiseKeys k, uint32_t j) { return mix32(j ^ k.k1) | 1u;
 FT_HD float noise_uniform(uint32_t a_i, uint32_t b_j) {
   uint32_t x = a_i * b_j;
   x ^= x >> 16;
+#if defined(__HIP_DEVICE_COMPILE__)
+  // (x >> 9) | 0x3f800000 in one v_alignbit_b32 is 1 + k 2^-23; subtracting 1 - 2^-24 leaves (k + 0.5) 2^-23,
+  // exactly, the value the arithmetic form below computes
+  return __builtin_bit_cast(float, __builtin_amdgcn_alignbit(0x7Fu, x, 9u)) - 0.99999994f;
+#else
   return (float)(x >> 9) * 1.1920928955078125e-07f + 5.9604644775390625e-08f;
+#endif
 }
+
+// log2(E) of E = -ln(u) = -ln2 * log2(u), as log2(-log2 u) + log2(ln 2): the constant is folded by callers
+constexpr float kLog2Ln2 = -0.5287663729448977f;
 
 }  // namespace ft
