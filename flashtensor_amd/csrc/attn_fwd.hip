@@ -66,7 +66,15 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // multiple of 8 a head stays on one XCD and its K/V are shared through that XCD's L2.  (Walking an XCD
   // through its heads one at a time cuts the K/V re-reads from 1.6x to 1.1x of the operand size but
   // loses the balance: measured 15% slower.)
-  const int mb = nMB - 1 - blockIdx.x / BH;
+  int mb = nMB - 1 - blockIdx.x / BH;
+  if (p.pair_order) {
+    // Every workgroup is resident from the start (no more of them than slots), so nothing is left to hand out
+    // as CUs free up: the heavy half is dealt first, descending, then the light half ascending, which tends to
+    // put a heavy and a light block on the same CU (measured 50 -> 47 us at B1 H32 S2048; with more
+    // workgroups than slots the descending order wins: 144 vs 164 us at S4096).
+    const int rank = blockIdx.x / BH, half = (nMB + 1) / 2;
+    mb = rank < half ? nMB - 1 - rank : rank - half;
+  }
   const int b = bh / p.H, h = bh % p.H;
   const int m0 = mb * BM;
   const int lane = lane_id(), wave = wave_id();
@@ -605,7 +613,9 @@ static int device_cu_count() {
 }
 
 template <typename T, int D, bool CAUSAL, bool EMU, int KF>
-static hipError_t launch_one(const AttnKernelParams& p, hipStream_t stream) {
+static hipError_t launch_one(const AttnKernelParams& p0, hipStream_t stream) {
+  AttnKernelParams p = p0;
+  p.pair_order = 0;
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
   // there are half as many of them: used on the pipelined fp16 paths once they still fill the chip twice
   constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast;
@@ -618,6 +628,7 @@ static hipError_t launch_one(const AttnKernelParams& p, hipStream_t stream) {
   }
   const int nMB = (p.Sq + 127) / 128;
   dim3 grid((unsigned)(nMB * p.B * p.H));
+  p.pair_order = CAUSAL && (int64_t)grid.x <= 2 * (int64_t)device_cu_count();  // two workgroups of this form per CU
   hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 4>), grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }

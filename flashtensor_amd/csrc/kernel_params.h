@@ -29,6 +29,7 @@ struct AttnKernelParams {
   // fp16 h except where |h / sqrt(D)| < 2.5e-3, and there within 2e-6 of it; both halves hold the constant
   uint32_t pk_hi2, pk_lo2;
   float softcap;    // kKfSoftcap: logits become softcap * tanh(logit / softcap)
+  int pair_order;   // block order of the causal attention kernel: heavy half descending, light half ascending
   int group;        // query heads per k/v head: query head h reads k/v head h / group
 };
 
