@@ -87,10 +87,10 @@ hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* 
     hipLaunchKernelGGL((topk_kernel<2, 256>), grid, dim3(256), 0, s, score, S, k, idx);
   else if (S <= 1024)
     hipLaunchKernelGGL((topk_kernel<4, 256>), grid, dim3(256), 0, s, score, S, k, idx);
-  else if (S <= 2048)
-    hipLaunchKernelGGL((topk_kernel<8, 256>), grid, dim3(256), 0, s, score, S, k, idx);
-  else if (S <= 4096)
-    hipLaunchKernelGGL((topk_kernel<16, 256>), grid, dim3(256), 0, s, score, S, k, idx);
+  else if (S <= 2048)  // more threads with fewer keys each beat fewer, fuller ones: 10.9 vs 12.9 us (8 keys x 256)
+    hipLaunchKernelGGL((topk_kernel<4, 512>), grid, dim3(512), 0, s, score, S, k, idx);
+  else if (S <= 4096)  // 21.3 vs 25.8 us (16 keys x 256)
+    hipLaunchKernelGGL((topk_kernel<8, 512>), grid, dim3(512), 0, s, score, S, k, idx);
   else
     hipLaunchKernelGGL((topk_kernel<16, 512>), grid, dim3(512), 0, s, score, S, k, idx);
   return hipGetLastError();
