@@ -523,6 +523,43 @@ def test_few_heads_rectangular_noncausal_grouped(gpu):
   assert (out_small.float() - out_big.float()).abs().max().item() <= 2e-3
 
 
+@pytest.mark.parametrize("S,Skv,D,causal,seed", [(4000, 4000, 128, True, 50), (3900, 4030, 128, True, 51), (3333, 3333, 64, True, 52),
+                                                 (3850, 520, 128, False, 53)])
+def test_large_ragged_shapes_256_row_blocks(gpu, S, Skv, D, causal, seed):
+  """Enough heads that the attention pass uses its 256-row (8-wave) workgroups, at sizes that leave ragged
+  last blocks and tiles, rectangular causal offsets and an unmasked problem; oracle on 2 of the 36 heads,
+  whole-problem invariants on all."""
+  H, HS = 36, 2
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, D, seed=seed, kv_len=Skv)
+  sub = tuple(t[:, :, :HS].contiguous() for t in (q, k, v))
+  if causal:
+    ref_o, r1, r2 = oracle.roco_forward(*sub)
+  else:
+    p = torch.softmax((torch.matmul(sub[0].transpose(1, 2), sub[1].transpose(1, 2).transpose(-2, -1)) / np.sqrt(D)).float(), -1)
+    ref_o, r1, r2 = torch.matmul(p.half(), sub[2].transpose(1, 2)).transpose(1, 2), p.sum(2), (p * p).sum(2)
+  out, s1, s2 = ops.roco(qd, kd, vd, causal=causal)
+  check_o(out[:, :, :HS], ref_o)
+  # The two sides accumulate QK^T in different orders; where a sum sits on an fp16 rounding boundary the logit
+  # comes out one ulp apart (up to 2^-8 for |logit| < 8) and that probability moves by as much.  A key seen by
+  # n rows carries such an element with weight <= 1 / n-ish, so the bar is 1e-3 + 4e-3 / n (twice that for the
+  # squares): the plain 1e-3 everywhere except on the last few keys of a causal problem.
+  n_rows = torch.full((Skv,), float(S))
+  if causal:
+    n_rows = (S - (torch.arange(Skv) - (Skv - S)).clamp_min(0)).float()
+  for got, ref, scale in ((s1, r1, 1.0), (s2, r2, 2.0)):
+    err = (got[:, :HS].float().cpu() - ref).abs() / ref.abs().clamp_min(1e-30)
+    assert (err <= scale * (1e-3 + 4e-3 / n_rows)).all(), f"score rel {err.max().item()}"
+  assert torch.allclose(s1.sum(-1).cpu(), torch.full((1, H), float(S)), rtol=1e-4)   # every row sums to one
+  # the same rows through the 128-row form (2 heads: too few workgroups for the 256-row form)
+  o2 = ops.attn(qd[:, :, :HS].contiguous(), kd[:, :, :HS].contiguous(), vd[:, :, :HS].contiguous(), causal=causal)
+  assert (out[:, :, :HS].float() - o2.float()).abs().max().item() <= 2e-3
+  if causal and D == 128:
+    check_o(ops.gemma2(qd, kd, vd)[:, :, :HS], oracle.gemma2_forward(*sub))
+    _, kf = ops.keyformer(qd, kd, vd, None, tau=1.0, seed=77)
+    es = oracle.seeded_exp_rand(77, 1, HS, S, Skv)
+    check_score(kf[:, :HS], oracle.keyformer_forward(*sub, es, tau=1.0)[1])
+
+
 # ------------------------------------------------------------------ grouped queries, 2-D harness form
 
 @pytest.mark.parametrize("S,Skv,H,Hkv,D,masked", [(128, 128, 4, 2, 128, True), (200, 200, 8, 2, 64, True), (96, 232, 4, 1, 128, True),
