@@ -30,6 +30,9 @@ def main():
   if args.model_name in cli.CASES_2D:
     fn = oracle.attn2d_forward if args.model_name == "attn_2d" else oracle.attn_h2o2d_forward
     ref = fn(*host, args.kv_head_num, args.head_num, args.head_dim, bool(args.masked))
+  elif args.model_name.endswith("_block"):
+    fn = oracle.ea_block_forward if args.model_name == "ea_block" else oracle.sima_block_forward
+    ref = fn(*host, args.head_num or 16)
   else:
     ref = ORACLE[args.model_name](*host)
   res = res if isinstance(res, tuple) else (res,)

@@ -666,3 +666,19 @@ def test_config5_ea_sima_b8_h16_s8192_d64(gpu):
   o16 = ops.sima(qd, kd, vd)
   ref16 = oracle.sima_forward(q, k, v)
   assert (o16.float().cpu() - ref16.float()).abs().max().item() <= 1.2e-7  # two fp16 subnormal steps
+
+
+# ------------------------------------------------------------------ command-line harness
+
+def test_cli_builds_and_runs_every_case(gpu, capsys):
+  from flashtensor_amd import run as cli
+  for name in sorted(ft.CASES) + sorted(cli.CASES_2D):
+    linear = name in ("ea", "sima", "ea_block", "sima_block")
+    argv = ["-m", name, "--q_len", "256", "--kv_len", "256", "--head_num", "4", "--head_dim", "64" if linear else "128",
+            "--run", "1", "--warmup", "1"]
+    if name in cli.CASES_2D:
+      argv += ["--kv_head_num", "2"]
+    res = cli.main(argv)
+    first = res[0] if isinstance(res, tuple) else res
+    assert torch.isfinite(first.float()).all(), name
+    assert "hip" in capsys.readouterr().out
