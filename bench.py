@@ -96,6 +96,15 @@ def per_config_table(dev):
   blk_bytes = (2.0 * M * C + 4 * C * C + 4 * C) * 2  # x in, y out, the weights and biases once
   add("5b ea block (projections + core)", "B8 S8192 C1024 H16", lambda: ops.ea_block(x, wq, bq, wo, bo, 16), blk_flops, blk_bytes)
   add("5b sima block", "B8 S8192 C1024 H16", lambda: ops.sima_block(x, wq, bq, wo, bo, 16, normalize_q=False), blk_flops, blk_bytes)
+  del x, wq, wo, bq, bo
+  # the literal shape of bench/ea.mlir:2 (x [64,784,128], 4 heads of 32), in fp16
+  C, M = 128, 64 * 784
+  x = torch.randn(64, 784, C, dtype=torch.float16, device=dev)
+  wq = (torch.randn(3 * C, C, device=dev) / C ** 0.5).half()
+  wo = (torch.randn(C, C, device=dev) / C ** 0.5).half()
+  bq, bo = torch.zeros(3 * C, dtype=torch.float16, device=dev), torch.zeros(C, dtype=torch.float16, device=dev)
+  add("5c ea block, .mlir shape", "B64 S784 C128 H4 D32", lambda: ops.ea_block(x, wq, bq, wo, bo, 4),
+      2 * 2.0 * 64 * 4 * 784 * 32 * 32 + 2.0 * M * 4 * C * C, (2.0 * M * C + 4 * C * C + 4 * C) * 2)
   return rows
 
 

@@ -422,7 +422,10 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Skv != a->Sq)
     return fail(FT_EINVAL, "bad shape B=%d H=%d Sq=%d Skv=%d (linear attention needs Sq == Skv)", a->B, a->H, a->Sq, a->Skv);
   if (a->Hkv != 0 && a->Hkv != a->H) return fail(FT_EUNSUPPORTED, "linear attention does not take grouped queries (H=%d Hkv=%d)", a->H, a->Hkv);
-  if (a->D != 64) return fail(FT_EUNSUPPORTED, "head_dim %d not supported by the linear-attention kernels (64)", a->D);
+  if (a->D != 64 && a->D != 32)
+    return fail(FT_EUNSUPPORTED, "head_dim %d not supported by the linear-attention kernels (64, or 32 in adjacent pairs)", a->D);
+  if (a->D == 32 && ((a->H & 1) || a->sq.h != 32 || a->sk.h != 32 || a->sv.h != 32 || a->so.h != 32))
+    return fail(FT_EUNSUPPORTED, "head_dim 32 needs an even number of heads stored 32 elements apart (H=%d)", a->H);
   if (a->dtype != FT_F16) return fail(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16)", a->dtype);
   if (out_dtype != FT_F16 && out_dtype != FT_F32) return fail(FT_EUNSUPPORTED, "out_dtype must be f16 or f32");
   if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->o))

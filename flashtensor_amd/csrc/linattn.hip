@@ -56,6 +56,7 @@ struct LinParams {
   int tiles_per_chunk;  // 128-token tiles per chunk of the K/V pass
   int out_nch;              // the same for the output pass (its chunks are independent of the K/V pass's)
   int out_tiles_per_chunk;
+  int half_heads;           // every 64-channel "head" is two adjacent heads of 32 channels (head_dim 32)
 };
 
 // Splits the sequence of every (b, h) into chunks so that about `workgroups` workgroups exist.  The K/V pass
@@ -67,7 +68,7 @@ constexpr int kKvWorkgroups = 512, kOutWorkgroups = 2048;
 
 static void lin_plan(const FtAttnArgs& a, int workgroups, int* nch, int* tpc) {
   const int ntiles = (a.Sq + kLinTile - 1) / kLinTile;
-  const int64_t bh = (int64_t)a.B * a.H;
+  const int64_t bh = (int64_t)a.B * a.H > 0 ? (int64_t)a.B * a.H : 1;
   int want = (int)((workgroups + bh - 1) / bh);
   if (want < 1) want = 1;
   int t = (ntiles + want - 1) / want;
@@ -77,7 +78,22 @@ static void lin_plan(const FtAttnArgs& a, int workgroups, int* nch, int* tpc) {
   *nch = (ntiles + t - 1) / t;
 }
 
-size_t linattn_workspace_bytes(const FtAttnArgs& a, int) {
+// head_dim 32 runs as head_dim 64 over pairs of adjacent heads (the caller has checked that H is even and that
+// the heads are 32 elements apart): the kernels see H / 2 heads of 64 channels and drop the cross-head blocks.
+static FtAttnArgs lin_effective(const FtAttnArgs& a0, int* half_heads) {
+  FtAttnArgs a = a0;
+  *half_heads = a0.D == 32;
+  if (*half_heads) {
+    a.H = a0.H / 2 > 0 ? a0.H / 2 : 1;  // sizes a workspace even for arguments the entry point will refuse
+    a.D = 64;
+    a.sq.h = a.sk.h = a.sv.h = a.so.h = 64;
+  }
+  return a;
+}
+
+size_t linattn_workspace_bytes(const FtAttnArgs& a0, int) {
+  int half;
+  const FtAttnArgs a = lin_effective(a0, &half);
   int nch, tpc;
   lin_plan(a, kKvWorkgroups, &nch, &tpc);
   const size_t bh = (size_t)a.B * a.H;
@@ -522,6 +538,9 @@ __global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinPar
   float gmax = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
+    // two heads of 32 channels side by side: the products between a channel of one and a channel of the other
+    // are not part of either head's matrix
+    if (p.half_heads && (drow[i] >> 5) != (qr >> 1)) accv[i] = 0.f;
     accv[i] *= s_scale[drow[i]];
     gmax = fmaxf(gmax, __builtin_fabsf(accv[i]));
   }
@@ -622,36 +641,46 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
 
     // EA: softmax over the 64 channels of the token.  The operand is the fp16 value of exp(q - max); the
     // division by the row sum (taken over those rounded values) is applied to the fp32 result.
-    float inv = 1.f;
+    // A lane holds channels 16 t + 8 g + [0..7]: t = 0, 1 lie in the first 32 channels, t = 2, 3 in the last 32.
+    // With head_dim 32 those are two heads, each with its own maximum and sum.
+    float inv[2] = {1.f, 1.f};
     if (EA) {
-      half2v hm = __builtin_shufflevector(qf[0], qf[0], 0, 1);
+      float mx[2], sum[2] = {0.f, 0.f};
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 0, 1));
-        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 2, 3));
-        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 4, 5));
-        hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 6, 7));
+      for (int hf = 0; hf < 2; ++hf) {
+        half2v hm = __builtin_shufflevector(qf[2 * hf], qf[2 * hf], 0, 1);
+#pragma unroll
+        for (int t = 2 * hf; t < 2 * hf + 2; ++t) {
+          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 0, 1));
+          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 2, 3));
+          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 4, 5));
+          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 6, 7));
+        }
+        mx[hf] = fmaxf((float)hm[0], (float)hm[1]);
       }
-      float mx = fmaxf((float)hm[0], (float)hm[1]);
-      mx = fmaxf(mx, xchg32(mx));
-      const float mb = mx * kLog2e;
+      if (!p.half_heads) mx[0] = mx[1] = fmaxf(mx[0], mx[1]);
+      mx[0] = fmaxf(mx[0], xchg32(mx[0]));
+      mx[1] = fmaxf(mx[1], xchg32(mx[1]));
       const half2v ones = {(_Float16)1.f, (_Float16)1.f};
-      float sum = 0.f;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
+        const float mb = mx[t >> 1] * kLog2e;
         uint4v pw;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float2v e2 = {__builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j], kLog2e, -mb)),
                               __builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j + 1], kLog2e, -mb))};
           const half2v ph = __builtin_convertvector(e2, half2v);
-          sum = __builtin_amdgcn_fdot2(ph, ones, sum, false);
+          sum[t >> 1] = __builtin_amdgcn_fdot2(ph, ones, sum[t >> 1], false);
           pw[j] = __builtin_bit_cast(uint32_t, ph);
         }
         qf[t] = __builtin_bit_cast(half8, pw);
       }
-      sum += xchg32(sum);
-      inv = 1.f / sum;
+      if (!p.half_heads) sum[0] = sum[1] = sum[0] + sum[1];
+      sum[0] += xchg32(sum[0]);
+      sum[1] += xchg32(sum[1]);
+      inv[0] = 1.f / sum[0];
+      inv[1] = 1.f / sum[1];
     }
 
     // W as hi + lo / 2^11 only where the output can show the difference (fp32)
@@ -672,7 +701,7 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
       }
     float osc[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) osc[i] = winv[i] * inv;
+    for (int i = 0; i < 4; ++i) osc[i] = winv[i] * inv[i >> 1];
 
     // accumulator (lane = token, registers = channels) -> padded [token][channel] rows in LDS
 #pragma unroll
@@ -719,8 +748,9 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
 }
 
 // ---------------------------------------------------------------------------------------------------
-hipError_t launch_linattn(const FtAttnArgs& a, int kind, int normalize_q, int out_dtype, void* ws, hipStream_t s) {
+hipError_t launch_linattn(const FtAttnArgs& a0, int kind, int normalize_q, int out_dtype, void* ws, hipStream_t s) {
   LinParams p;
+  const FtAttnArgs a = lin_effective(a0, &p.half_heads);
   p.q = (const uint16_t*)a.q;
   p.k = (const uint16_t*)a.k;
   p.v = (const uint16_t*)a.v;

@@ -155,7 +155,8 @@ int check_block(const FtLinBlockArgs* b, int kind) {
   if (!b) return ft::set_error(FT_EINVAL, "args is null");
   if (kind != FT_OP_EA && kind != FT_OP_SIMA) return ft::set_error(FT_EINVAL, "kind must be FT_OP_EA or FT_OP_SIMA");
   if (b->B < 1 || b->S < 1 || b->H < 1) return ft::set_error(FT_EINVAL, "bad shape B=%d S=%d H=%d", b->B, b->S, b->H);
-  if (b->D != 64) return ft::set_error(FT_EUNSUPPORTED, "head_dim %d not supported by the linear-attention kernels (64)", b->D);
+  if (b->D != 64 && !(b->D == 32 && (b->H & 1) == 0))
+    return ft::set_error(FT_EUNSUPPORTED, "head_dim %d with %d heads not supported by the linear-attention kernels (64, or 32 with an even number of heads)", b->D, b->H);
   if (b->dtype != FT_F16) return ft::set_error(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16)", b->dtype);
   return FT_OK;
 }

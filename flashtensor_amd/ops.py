@@ -177,6 +177,8 @@ def gemma2(q, k, v, softcap=50.0, causal=True, fast_logits=False):
 
 def _linattn(q, k, v, kind, normalize_q, out_dtype):
   q, k, v = _prep(q, k, v)
+  if q.shape[3] == 32:  # head_dim 32 runs as pairs of adjacent heads: heads must lie 32 elements apart
+    q, k, v = (t if t.stride(2) == 32 else t.contiguous() for t in (q, k, v))
   lib = _lib.load()
   out_dtype = out_dtype or q.dtype
   if out_dtype not in (torch.float16, torch.float32):

@@ -117,7 +117,8 @@ int ft_avgpool1d(const float* src, int64_t rows, int32_t S, int32_t kernel, floa
 
 /* Linear attention cores of bench/ea.mlir:13-17 (kind = FT_OP_EA) and bench/sima.mlir:13-17 (FT_OP_SIMA):
  * O = f(Q) (g(K)^T V).  normalize_q applies SimA's L1 normalisation to Q as well (ignored for EA).
- * out_dtype: FtDtype of o (FT_F16/FT_BF16 = a->dtype, or FT_F32). */
+ * out_dtype: FtDtype of o (FT_F16/FT_BF16 = a->dtype, or FT_F32).  fp16 inputs; head_dim 64, or 32 (the
+ * .mlir's own 4 heads of 32, :7-9) with an even number of heads stored 32 elements apart (s*.h == 32). */
 int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype, void* workspace,
                    size_t workspace_bytes, void* stream);
 
@@ -125,7 +126,8 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
  * qkv = x w_qkv^T + b_qkv (w_qkv [3C,C] row-major as in a Linear, :3-5), split into q, k, v and into heads
  * (:6-12), the core (:13-17), y = core w_out^T + b_out (w_out [C,C], :20-22).  All tensors 16-bit and
  * contiguous; biases may be NULL.  The two projections are hipBLASLt GEMMs (fp32 accumulation, bias added
- * before the one rounding to 16 bits); q/k/v and the core's result live in the workspace as 16-bit tensors. */
+ * before the one rounding to 16 bits); q/k/v and the core's result live in the workspace as 16-bit tensors.
+ * fp16; D = 64, or 32 with an even H. */
 typedef struct FtLinBlockArgs {
   const void* x;
   const void* w_qkv;

@@ -120,6 +120,14 @@ def test_linattn_and_topk_argument_checks(lib):
   assert lib.ft_linattn_fwd(ctypes.byref(a), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
   b = _args(D=128, flags=0)
   assert lib.ft_linattn_fwd(ctypes.byref(b), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EUNSUPPORTED
+  st32 = FtStrides(64 * 4 * 32, 4 * 32, 32)
+  d32 = _args(D=32, H=4, Sq=64, Skv=64, sq=st32, sk=st32, sv=st32, so=st32, flags=0)
+  need32 = lib.ft_workspace_bytes(_lib.FT_OP_SIMA, ctypes.byref(d32))
+  assert need32 > 0 and lib.ft_linattn_fwd(ctypes.byref(d32), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, need32 - 1, None) == _lib.FT_EWORKSPACE
+  odd = _args(D=32, H=3, Sq=64, Skv=64, sq=st32, sk=st32, sv=st32, so=st32, flags=0)
+  assert lib.ft_linattn_fwd(ctypes.byref(odd), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EUNSUPPORTED
+  far = _args(D=32, H=4, Sq=64, Skv=64, sq=st, sk=st, sv=st, so=st, flags=0)   # heads 64 apart: not adjacent pairs
+  assert lib.ft_linattn_fwd(ctypes.byref(far), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EUNSUPPORTED
   c = _args(D=64, Sq=64, Skv=32, sq=st, sk=st, sv=st, so=st, flags=0)
   assert lib.ft_linattn_fwd(ctypes.byref(c), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EINVAL
   assert lib.ft_topk(None, 1, 8, 2, 0x1000, None) == _lib.FT_EINVAL
@@ -135,9 +143,14 @@ def test_linear_block_argument_checks(lib):
   assert lib.ft_linattn_block_fwd(ctypes.byref(b), _lib.FT_OP_EA, 1, 0x10000, need - 1, None) == _lib.FT_EWORKSPACE
   assert lib.ft_linattn_block_fwd(ctypes.byref(b), 9, 1, 0x10000, need, None) == _lib.FT_EINVAL
   assert lib.ft_linattn_block_fwd(None, _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
-  bad = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 32, _lib.FT_F16)
+  bad = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 48, _lib.FT_F16)
   assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(bad), _lib.FT_OP_EA) == 0
   assert "head_dim" in lib.ft_last_error().decode()
+  # head_dim 32 runs as pairs of adjacent heads: an even number of them
+  d32 = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 32, _lib.FT_F16)
+  assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(d32), _lib.FT_OP_EA) > 0
+  odd32 = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 3, 32, _lib.FT_F16)
+  assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(odd32), _lib.FT_OP_SIMA) == 0
   assert lib.ft_linattn_block_fwd(ctypes.byref(bad), _lib.FT_OP_SIMA, 1, 0x10000, need, None) == _lib.FT_EUNSUPPORTED
   odd = _lib.FtLinBlockArgs(0x1008, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
   assert lib.ft_linattn_block_fwd(ctypes.byref(odd), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL

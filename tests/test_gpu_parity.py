@@ -306,6 +306,40 @@ def test_ea_sima_small(gpu, B, S, H, seed):
   assert (o16.float().cpu() - ref32.half().float()).abs().max().item() <= max(6e-8, 1e-3 * ref32.abs().max().item())
 
 
+@pytest.mark.parametrize("B,S,H,seed", [(2, 200, 4, 20), (1, 333, 2, 21), (1, 784, 6, 22), (1, 1, 2, 23)])
+def test_ea_sima_head_dim_32(gpu, B, S, H, seed):
+  """head_dim 32 (the literal shape of bench/ea.mlir:7-9) runs as pairs of adjacent heads on the 64-channel
+  kernels; nothing of one head may leak into its neighbour."""
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, 32, seed=seed)
+  check_o(ops.ea(qd, kd, vd), oracle.ea_forward(q, k, v))
+  check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), oracle.sima_forward(q, k, v, out_dtype=torch.float32))
+  check_sima(ops.sima(qd, kd, vd, normalize_q=False, out_dtype=torch.float32),
+             oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32))
+  # changing one head's inputs leaves the other heads' outputs bit-identical
+  q2, k2, v2 = qd.clone(), kd.clone(), vd.clone()
+  q2[:, :, 1], k2[:, :, 1], v2[:, :, 1] = q2[:, :, 1] * 3 + 1, k2[:, :, 1] * -2, v2[:, :, 1] + 5
+  a, b = ops.ea(qd, kd, vd), ops.ea(q2, k2, v2)
+  assert torch.equal(a[:, :, 0], b[:, :, 0]) and not torch.equal(a[:, :, 1], b[:, :, 1])
+  # a [B,H,S,D] storage order is made head-adjacent by the binding
+  qt = qd.transpose(1, 2).contiguous().transpose(1, 2)
+  assert torch.equal(ops.ea(qt, kd, vd), a)
+  with pytest.raises(RuntimeError, match="even number of heads"):
+    ops.ea(qd[:, :, :1].contiguous(), kd[:, :, :1].contiguous(), vd[:, :, :1].contiguous())
+
+
+def test_linear_block_mlir_literal_shape(gpu):
+  """bench/ea.mlir:2 and bench/sima.mlir:2 as written: x [64, 784, 128], 4 heads of 32 (in fp16 here); the
+  oracle on 3 of the 64 batches."""
+  B, S, H, D = 64, 784, 4, 32
+  host, dev = block_inputs(gpu, B, S, H, D, seed=6)
+  y = ops.ea_block(*dev, H)
+  ys = ops.sima_block(*dev, H, normalize_q=False)
+  for b in (0, 31, 63):
+    hb = (host[0][b:b + 1],) + host[1:]
+    check_o(y[b:b + 1], oracle.ea_block_forward(*hb, H))
+    check_o(ys[b:b + 1], oracle.sima_block_forward(*hb, H, normalize_q=False))
+
+
 def test_ea_sima_properties(gpu):
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 512, 2, 64, seed=5)
   c = torch.full_like(vd, 0.75)
@@ -359,7 +393,7 @@ def test_linear_block_properties(gpu):
   with pytest.raises(ValueError, match="weights need"):
     ops.ea_block(x, wq[:C], bq, wo, bo, H)
   with pytest.raises(RuntimeError, match="head_dim"):
-    ops.ea_block(x, wq, bq, wo, bo, 4)
+    ops.ea_block(x, wq, bq, wo, bo, 8)   # head_dim 16
 
 
 def test_linear_block_config5_shape(gpu):

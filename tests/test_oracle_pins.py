@@ -141,6 +141,13 @@ def test_ea_closed_forms_and_brute_force():
   assert (got - ref.expand_as(got)).abs().max() < 1e-3
 
 
+def test_linear_cores_head_dim_32_brute_force():
+  q, k, v = _inputs(B=1, S=33, H=3, D=32, seed=12)
+  assert np.abs(oracle.ea_forward(q, k, v).float().numpy() - brute.ea(q, k, v)).max() < 2e-3
+  ref = brute.sima(q, k, v)
+  assert np.abs(oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy() - ref).max() / np.abs(ref).max() < 1e-5
+
+
 def test_sima_invariants_and_brute_force():
   q, k, v = _inputs(B=1, S=40, H=2, D=64, seed=6)
   out32 = oracle.sima_forward(q, k, v, out_dtype=torch.float32)
