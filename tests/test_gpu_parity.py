@@ -702,6 +702,48 @@ def test_config5_ea_sima_b8_h16_s8192_d64(gpu):
   assert (o16.float().cpu() - ref16.float()).abs().max().item() <= 1.2e-7  # two fp16 subnormal steps
 
 
+# ------------------------------------------------------------------ HIP graph capture
+
+def test_calls_can_be_captured_in_a_hip_graph(gpu):
+  """The entry points only queue kernels on the stream they are given (no allocation, no memset, no
+  synchronisation), so a caller may record them into a HIP graph: several replays with fresh inputs, eager
+  work in between, every replay compared with the eager result."""
+  B, S, H, D = 1, 512, 4, 128
+  static = [torch.zeros(B, S, H, D, dtype=torch.float16, device=gpu) for _ in range(3)]
+  xs = torch.zeros(2, 300, 2 * 64, dtype=torch.float16, device=gpu)
+  _, blk = block_inputs(gpu, 2, 300, 2, 64, seed=3)
+
+  def work():
+    out, score = ops.h2o(*static)
+    idx = ops.topk(score, S // 8)
+    _, kf = ops.keyformer(*static, None, tau=1.0, seed=5)
+    lin = ops.ea(static[0][..., :64], static[1][..., :64], static[2][..., :64])
+    y = ops.ea_block(xs, *blk[1:], 2)
+    return out, score, idx, kf, lin, y
+
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    work()                                   # warm-up outside the capture (lazy initialisation, GEMM plans)
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    captured = work()
+  for seed in (31, 32, 33):
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+    for dst, src in zip(static, (q, k, v)):
+      dst.copy_(src.to(gpu))
+    xs.copy_(torch.randn(2, 300, 128, generator=torch.Generator().manual_seed(seed)).half().to(gpu))
+    graph.replay()
+    torch.cuda.synchronize()
+    got = [t.clone() for t in captured]
+    eager = work()                           # the program's own eager work between replays
+    torch.cuda.synchronize()
+    for g, e in zip(got, eager):
+      assert torch.equal(g, e)
+
+
 # ------------------------------------------------------------------ command-line harness
 
 def test_cli_builds_and_runs_every_case(gpu, capsys):
