@@ -29,8 +29,6 @@ constexpr int kAttnBN = 64;
 // below 2^kRescaleSlack (exact in fp16/fp32; the final division uses the same maximum).
 constexpr float kRescaleSlack = 6.f;
 
-enum TileMode { kTileFast = 0, kTileMasked = 1, kTileIdle = 2 };
-
 template <typename T, int D, bool CAUSAL, bool EMU, int KF, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const AttnKernelParams p) {
   constexpr int BM = 32 * WAVES, BN = kAttnBN, NT = 64 * WAVES;
@@ -101,7 +99,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     nw = min(ntiles, (wave_row0 + 31 + p.off) / BN + 1);
     n_fast = min(n_fast, (wave_row0 + p.off + 1) / BN);  // tiles with n0 + BN - 1 <= wave_row0 + off
   }
-  if (!kFastMasked) n_fast = 0;  // only the packed fp16 path has a mask-free instance
+  if (!kFastMasked) n_fast = 0;  // only the pipelined path has a mask-free instance
   n_fast = min(n_fast, nw);
 
   NoiseKeys nk = {0, 0};
@@ -203,7 +201,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     }
   };
 
-  // ---- mask-free fp16 softmax, in two parts so that the rescale branch sits between them.
+  // ---- softmax of the pipelined path, in two parts so that the rescale branch sits between them.
   // Rounding is monotonic, so the row maximum of the rounded logits is the rounded maximum of the raw
   // accumulators.
   // MASKED (tiles that straddle the diagonal or the end of K): hidden keys are left out of the maximum, so
@@ -351,84 +349,81 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // ---- softmax of one tile: s (raw accumulators) -> pb (16-bit unnormalised probabilities)
   auto softmax = [&](auto masked_tag, float16v (&s)[2], vec8 (&pb)[4], int n0, int buf, const float (&er)[2][16]) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    if constexpr (false) {
-    } else {
-      // ---- logits in the log2 domain, with the reference's rounding points when EMU
-      const int jmax = CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1;  // last key this query sees
-      float rowmax = NEG_INF;
+    // ---- logits in the log2 domain, with the reference's rounding points when EMU
+    const int jmax = CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1;  // last key this query sees
+    float rowmax = NEG_INF;
+#pragma unroll
+    for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float x = s[mbk][r];
+        if (EMU) {
+          x = T::to_float(T::from_float(x));
+          x = T::to_float(T::from_float(x * p.logit_mul));
+          if (KF == kKfSoftcap) {  // three 16-bit tensor ops in the reference (cases/kernels/gemma2.py:31-33)
+            x = T::to_float(T::from_float(x / p.softcap));
+            x = T::to_float(T::from_float(tanh_f32(x)));
+            x = T::to_float(T::from_float(x * p.softcap));
+          }
+          x *= kLog2e;
+        } else if (KF == kKfSoftcap) {
+          x = p.softcap * tanh_f32(x * (p.logit_mul * (1.f / kLog2e)) / p.softcap) * kLog2e;
+        } else {
+          x *= p.logit_mul;
+        }
+        if (MASKED) {
+          const int j = n0 + 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
+          x = (j > jmax) ? NEG_INF : x;
+        }
+        s[mbk][r] = x;
+        rowmax = fmaxf(rowmax, x);
+      }
+    rowmax = fmaxf(rowmax, xchg32(rowmax));
+
+    // ---- KeyFormer: running normaliser of softmax((logit + gumbel) / tau), gumbel = -ln(E)
+    if (KF == kKfTensor || KF == kKfSeeded) {
+      float z[2][16];
+      float zmax = NEG_INF;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          float x = s[mbk][r];
-          if (EMU) {
-            x = T::to_float(T::from_float(x));
-            x = T::to_float(T::from_float(x * p.logit_mul));
-            if (KF == kKfSoftcap) {  // three 16-bit tensor ops in the reference (cases/kernels/gemma2.py:31-33)
-              x = T::to_float(T::from_float(x / p.softcap));
-              x = T::to_float(T::from_float(tanh_f32(x)));
-              x = T::to_float(T::from_float(x * p.softcap));
-            }
-            x *= kLog2e;
-          } else if (KF == kKfSoftcap) {
-            x = p.softcap * tanh_f32(x * (p.logit_mul * (1.f / kLog2e)) / p.softcap) * kLog2e;
+          float log2E;
+          if (KF == kKfTensor) {
+            log2E = __builtin_amdgcn_logf(er[mbk][r]);
           } else {
-            x *= p.logit_mul;
+            const int jl = 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
+            const float u = noise_uniform(a_i, ldsCol[buf * BN + jl]);
+            log2E = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(u));
           }
-          if (MASKED) {
-            const int j = n0 + 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
-            x = (j > jmax) ? NEG_INF : x;
-          }
-          s[mbk][r] = x;
-          rowmax = fmaxf(rowmax, x);
+          const float zz = (s[mbk][r] - log2E) * p.inv_tau;
+          z[mbk][r] = zz;
+          zmax = fmaxf(zmax, zz);
         }
-      rowmax = fmaxf(rowmax, xchg32(rowmax));
-
-      // ---- KeyFormer: running normaliser of softmax((logit + gumbel) / tau), gumbel = -ln(E)
-      if (KF == kKfTensor || KF == kKfSeeded) {
-        float z[2][16];
-        float zmax = NEG_INF;
-#pragma unroll
-        for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float log2E;
-            if (KF == kKfTensor) {
-              log2E = __builtin_amdgcn_logf(er[mbk][r]);
-            } else {
-              const int jl = 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
-              const float u = noise_uniform(a_i, ldsCol[buf * BN + jl]);
-              log2E = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(u));
-            }
-            const float zz = (s[mbk][r] - log2E) * p.inv_tau;
-            z[mbk][r] = zz;
-            zmax = fmaxf(zmax, zz);
-          }
-        zmax = fmaxf(zmax, xchg32(zmax));
-        const float mk_new = fmaxf(m_kf, zmax);
-        float zs = 0.f;
-#pragma unroll
-        for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) zs += __builtin_amdgcn_exp2f(z[mbk][r] - mk_new);
-        l_kf = l_kf * __builtin_amdgcn_exp2f(m_kf - mk_new) + zs;
-        m_kf = mk_new;
-      }
-
-      rescale(rowmax);
-      uint4v pw[4];
+      zmax = fmaxf(zmax, xchg32(zmax));
+      const float mk_new = fmaxf(m_kf, zmax);
+      float zs = 0.f;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const uint16_t b0 = T::from_float(__builtin_amdgcn_exp2f(s[mbk][r] - m_run));
-          const uint16_t b1 = T::from_float(__builtin_amdgcn_exp2f(s[mbk][r + 1] - m_run));
-          l_run += T::to_float(b0) + T::to_float(b1);
-          pw[2 * mbk + (r >> 3)][(r & 7) >> 1] = (uint32_t)b0 | ((uint32_t)b1 << 16);
-        }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
+        for (int r = 0; r < 16; ++r) zs += __builtin_amdgcn_exp2f(z[mbk][r] - mk_new);
+      l_kf = l_kf * __builtin_amdgcn_exp2f(m_kf - mk_new) + zs;
+      m_kf = mk_new;
     }
+
+    rescale(rowmax);
+    uint4v pw[4];
+#pragma unroll
+    for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const uint16_t b0 = T::from_float(__builtin_amdgcn_exp2f(s[mbk][r] - m_run));
+        const uint16_t b1 = T::from_float(__builtin_amdgcn_exp2f(s[mbk][r + 1] - m_run));
+        l_run += T::to_float(b0) + T::to_float(b1);
+        pw[2 * mbk + (r >> 3)][(r & 7) >> 1] = (uint32_t)b0 | ((uint32_t)b1 << 16);
+      }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
   };
 
   // ---- O^T += V^T P^T (32 transposed LDS reads, 16 MFMAs)
@@ -460,7 +455,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
   };
 
-  // One tile of the pipelined loop (fp16, reference rounding): the QK^T MFMAs of the next tile and the PV
+  // One tile of the pipelined loop: the QK^T MFMAs of the next tile and the PV
   // MFMAs of this tile are spread over this tile's softmax VALU instructions (only about four hide
   // behind one MFMA, so the two kinds are interleaved as finely as the dependencies allow).  The first
   // half of QK^T covers the latency of the row-maximum reduction and of the (rare) rescale branch.
@@ -617,7 +612,7 @@ static hipError_t launch_one(const AttnKernelParams& p0, hipStream_t stream) {
   AttnKernelParams p = p0;
   p.pair_order = 0;
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
-  // there are half as many of them: used on the pipelined fp16 paths once they still fill the chip twice
+  // there are half as many of them: used on the pipelined paths once they still fill the chip twice
   constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast;
   if constexpr (kHas8) {
     const int64_t n8 = (int64_t)((p.Sq + 255) / 256) * p.B * p.H;

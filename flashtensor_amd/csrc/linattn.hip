@@ -1,4 +1,5 @@
-// Linear-attention cores EA and SimA for gfx950, head_dim 64, fp16.
+// Linear-attention cores EA and SimA for gfx950, fp16, head_dim 64 (head_dim 32 as pairs of adjacent heads:
+// the merge step drops the two cross-head blocks of the 64x64 matrix, the output step keeps EA's softmax per half).
 //
 // Replaces the fused kernels the reference would emit for bench/ea.mlir:13-17 and bench/sima.mlir:13-17
 // (asuka.softmax / asuka.normalize semantics: lib/Dialect/Asuka/Transforms/LowerComplexReduce.cpp:21-69):
