@@ -43,8 +43,9 @@ def event_time_us(fn, iters, warmup=20):
   return start.elapsed_time(end) * 1e3 / iters
 
 
-def per_config_table(dev):
-  """µs per call, algorithmic TFLOP/s and GB/s with their roofline fractions for the five configurations."""
+def per_config_table(dev, only=None, iters=100):
+  """µs per call, algorithmic TFLOP/s and GB/s with their roofline fractions for the five configurations
+  (`only`: just the rows whose name contains that text)."""
   import torch
   from flashtensor_amd import ops
   rows = []
@@ -52,7 +53,9 @@ def per_config_table(dev):
   def qkv(B, S, H, D):
     return tuple(torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3))
 
-  def add(name, shape, fn, flops, nbytes, iters=100):
+  def add(name, shape, fn, flops, nbytes):
+    if only is not None and only not in name:
+      return
     us = event_time_us(fn, iters)
     tf, gb = flops / us / 1e6, nbytes / us / 1e3
     rows.append({"config": name, "shape": shape, "us": round(us, 1), "tflops": round(tf, 1),
@@ -68,10 +71,11 @@ def per_config_table(dev):
   softmax_case("2' h2o", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.h2o(q, k, v)), extra_bytes=32 * 4096 * 4)
   softmax_case("3 keyformer seeded tau=1", 1, 4096, 32, 128,
                lambda q, k, v: (lambda: ops.keyformer(q, k, v, None, tau=1.0, seed=1)), extra_bytes=32 * 4096 * 4)
-  er = 1 + torch.randn(1, 32, 4096, 4096, dtype=torch.float32, device=dev).abs()
-  softmax_case("3t keyformer tensor noise tau=1.5", 1, 4096, 32, 128,
-               lambda q, k, v: (lambda: ops.keyformer(q, k, v, er, tau=1.5)), extra_bytes=2 * er.numel() * 4)
-  del er
+  if only is None or only in "3t keyformer tensor noise tau=1.5":
+    er = 1 + torch.randn(1, 32, 4096, 4096, dtype=torch.float32, device=dev).abs()
+    softmax_case("3t keyformer tensor noise tau=1.5", 1, 4096, 32, 128,
+                 lambda q, k, v: (lambda: ops.keyformer(q, k, v, er, tau=1.5)), extra_bytes=2 * er.numel() * 4)
+    del er
   softmax_case("4 roco", 4, 4096, 32, 128, lambda q, k, v: (lambda: ops.roco(q, k, v)), extra_bytes=2 * 4 * 32 * 4096 * 4)
   # the other cases of the reference's zoo at their prepare() defaults (B=1 H=32 S=4096 D=128)
   softmax_case("snapkv k=5", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.snapkv(q, k, v)), extra_bytes=32 * 4096 * 4)
@@ -131,6 +135,8 @@ def main():
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
   ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
   ap.add_argument("--cpu-heads", type=int, default=4)
+  ap.add_argument("--only", default=None, help="per-configuration table: only the rows whose name contains this text")
+  ap.add_argument("--config-iters", type=int, default=100, help="timed calls per row of the per-configuration table")
   ap.add_argument("--calibrate-copy", action="store_true",
                   help="also run a 256 MiB device-to-device tensor copy a few times: under rocprofv3 --pmc its "
                        "FETCH_SIZE / WRITE_SIZE readings give the counter unit for the other kernels")
@@ -202,7 +208,7 @@ def main():
                      "step_events": round(step_us, 1)},
   }
   if not args.no_configs:
-    result["per_config"] = per_config_table(dev)
+    result["per_config"] = per_config_table(dev, args.only, args.config_iters)
   if not args.no_cpu:
     result["cpu_baseline"] = cpu_baseline(B, S, H, D, args.cpu_heads)
   else:

@@ -298,7 +298,8 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
   };
 
   // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P
-  // (always fetched: rows are clamped), then consume the parked strip
+  // if this wave has one (a strip past its share would be another workgroup's rows: wasted HBM reads), then
+  // consume the parked strip
   auto step = [&](int i, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     const int t0 = strip_row0(i);
@@ -316,7 +317,7 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
         for (int e = 0; e < 8; ++e) qabs[e] += live ? __builtin_fabsf((float)qv[e]) : 0.f;
       }
     }
-    fetch(i + P, slot_tag);
+    if (i + P < nmine) fetch(i + P, slot_tag);
     wave_lds_order();
     if (tail)
       compute(std::true_type{}, t0);
@@ -324,9 +325,9 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
       compute(std::false_type{}, t0);
   };
 
-  fetch(0, std::integral_constant<int, 0>{});
-  fetch(1, std::integral_constant<int, 1>{});
-  fetch(2, std::integral_constant<int, 2>{});
+  if (0 < nmine) fetch(0, std::integral_constant<int, 0>{});
+  if (1 < nmine) fetch(1, std::integral_constant<int, 1>{});
+  if (2 < nmine) fetch(2, std::integral_constant<int, 2>{});
   static_assert(P == 3, "the strip loop is unrolled over three register slots");
   for (int i = 0; i < nmine;) {
     step(i, std::integral_constant<int, 0>{});
@@ -605,8 +606,8 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
   uint4v rq[P][R];  // strips in flight, indexed by compile-time slot
   auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * SUB; };
-  mvQ.load(strip_row0(0), rq[0]);
-  mvQ.load(strip_row0(1), rq[1]);
+  if (0 < nmine) mvQ.load(strip_row0(0), rq[0]);
+  if (1 < nmine) mvQ.load(strip_row0(1), rq[1]);
 
   // A operand: W^T[e][d], hi and lo, rows e = 32 eb + n, contraction slots d = 16 t + 8 g + [0..7]
   const uint16_t* w = p.w + (int64_t)bh * 2 * D * D;
@@ -626,13 +627,14 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   const int64_t orow_bytes = p.so.s * (int64_t)(F32OUT ? 4 : 2);
 
   // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P
-  // (always fetched: rows are clamped), then consume the parked strip
+  // if this wave has one (a strip past its share would be another workgroup's rows: wasted HBM reads), then
+  // consume the parked strip
   auto step = [&](int i, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     const int t0 = strip_row0(i);
     wave_lds_order();
     mvQ.to_lds(rq[SLOT], tq);
-    mvQ.load(strip_row0(i + P), rq[SLOT]);
+    if (i + P < nmine) mvQ.load(strip_row0(i + P), rq[SLOT]);
     wave_lds_order();
 
     // B operand: f(Q)^T, column = token n, same contraction slots
