@@ -241,14 +241,22 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
         mx = fmaxf(mx, xchg32(mx));
         m_new[db] = fmaxf(m_run[db], mx);
       }
-      if (__any(m_new[0] > m_run[0] || m_new[1] > m_run[1])) {
+      // Lazy: the stale maximum is kept while no channel has outgrown it by more than kStaleMax (the operand
+      // exp(k - m) then stays below e^4 = 55, exact enough in fp16 and far from its range; sums and matrix are
+      // fp32 and the merge step works with whatever maximum a chunk reports).  Without the slack some of the
+      // 64 channels moves its maximum in almost every strip and the whole 64x64 matrix is rescaled each time.
+      constexpr float kStaleMax = 4.f;
+      if (__any(m_new[0] > m_run[0] + kStaleMax || m_new[1] > m_run[1] + kStaleMax)) {
         // move the per-channel factor from "lane = channel" to the accumulator's "register = channel"
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
-          const float f = __builtin_amdgcn_exp2f((m_run[db] - m_new[db]) * kLog2e);
+          // only the channels that outgrew their maximum move (factor exactly 1 for the others), so a channel's
+          // arithmetic depends on its own column of K alone
+          const float mt = m_new[db] > m_run[db] + kStaleMax ? m_new[db] : m_run[db];
+          const float f = __builtin_amdgcn_exp2f((m_run[db] - mt) * kLog2e);
           l_run[db] *= f;
           if (g == 0) fac[32 * db + n] = f;
-          m_run[db] = m_new[db];
+          m_run[db] = mt;
         }
         wave_lds_order();
 #pragma unroll
