@@ -22,6 +22,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SHAPES = [("s128_d128", 1, 128, 2, 128, 0), ("s256_d64", 1, 256, 2, 64, 0), ("s200_d128", 1, 200, 2, 128, 1)]
 LIN_SHAPES = [("s256_d64", 1, 256, 2, 64, 0), ("s200_d64", 2, 200, 2, 64, 1)]
 NEXT_SHAPES = [("s128_d128", 1, 128, 2, 128, 3), ("s200_d64", 1, 200, 4, 64, 4)]
+BLOCK_SHAPES = [("s200_h2_d64", 2, 200, 2, 64, 5), ("s150_h4_d32", 1, 150, 4, 32, 6)]  # the second: head_dim 32, the .mlir's own
 KF_SEED = 1234
 
 
@@ -55,6 +56,14 @@ def main():
                         gemma2_cap50=oracle.gemma2_forward(q, k, v).numpy(),
                         gemma2_cap2=oracle.gemma2_forward(q, k, v, softcap=2.0).numpy(),
                         gqa_out=og.numpy(), gqa_score=sg.numpy())
+  for name, B, S, H, D, seed in BLOCK_SHAPES:
+    args = oracle.prepare_block_inputs(B, S, H, D, seed=seed)
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+    np.savez_compressed(os.path.join(HERE, f"block_{name}.npz"), B=B, S=S, H=H, D=D, seed=seed,
+                        ea_block=oracle.ea_block_forward(*args, H).numpy(),
+                        sima_block_rawq=oracle.sima_block_forward(*args, H, normalize_q=False).numpy(),
+                        ea_core=oracle.ea_forward(q, k, v).numpy(),
+                        sima_core=oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy())
   print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
 
 

@@ -224,6 +224,18 @@ def test_linear_golden(gpu, path):
   check_sima(ops.sima(qd, kd, vd, normalize_q=False, out_dtype=torch.float32), torch.from_numpy(g["sima_rawq"]))
 
 
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "block_*.npz"))), ids=os.path.basename)
+def test_block_golden(gpu, path):
+  g = np.load(path, allow_pickle=False)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  dev = tuple(t.to(gpu) for t in oracle.prepare_block_inputs(B, S, H, D, seed=seed))
+  check_o(ops.ea_block(*dev, H), torch.from_numpy(g["ea_block"]))
+  check_o(ops.sima_block(*dev, H, normalize_q=False), torch.from_numpy(g["sima_block_rawq"]))
+  _, (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed)
+  check_o(ops.ea(qd, kd, vd), torch.from_numpy(g["ea_core"]))
+  check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), torch.from_numpy(g["sima_core"]))
+
+
 def check_sima(out, ref, rel=1e-3):
   """SimA outputs are ~1e-5 (fp16-subnormal range): compare in fp32 relative to the largest reference
   magnitude; the fp16 output is checked against the fp16 rounding of the reference."""

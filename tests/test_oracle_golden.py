@@ -63,5 +63,18 @@ def test_next_cases_match_golden(path):
   np.testing.assert_allclose(sg.numpy(), g["gqa_score"], rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "block_*.npz"))), ids=os.path.basename)
+def test_block_cases_match_golden(path):
+  g = _load(path)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  args = oracle.prepare_block_inputs(B, S, H, D, seed=seed)
+  assert np.abs(oracle.ea_block_forward(*args, H).float().numpy() - g["ea_block"].astype(np.float32)).max() <= 2e-3
+  assert np.abs(oracle.sima_block_forward(*args, H, normalize_q=False).float().numpy()
+                - g["sima_block_rawq"].astype(np.float32)).max() <= 2e-3
+  q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+  assert np.abs(oracle.ea_forward(q, k, v).float().numpy() - g["ea_core"].astype(np.float32)).max() <= 1e-3
+  np.testing.assert_allclose(oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy(), g["sima_core"], rtol=1e-4, atol=1e-9)
+
+
 def test_golden_files_present():
-  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 7
+  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 9
