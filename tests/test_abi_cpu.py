@@ -158,6 +158,33 @@ def test_linear_block_argument_checks(lib):
   assert lib.ft_linattn_block_fwd(ctypes.byref(nul), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
 
 
+def test_last_error_is_per_thread(lib):
+  import threading
+  seen, barrier = {}, threading.Barrier(4)
+
+  def worker(i):
+    barrier.wait()
+    for _ in range(200):
+      if i % 2:
+        rc = lib.ft_topk(0x1000, 1, 8, 9 + i, 0x2000, None)           # k > S
+        want = f"k={9 + i}"
+      else:
+        rc = lib.ft_avgpool1d(0x1000, 1, 8, 4 + i, 0x2000, None)      # even window
+        want = "odd"
+      msg = lib.ft_last_error().decode()
+      if rc != _lib.FT_EINVAL or want not in msg:
+        seen[i] = (rc, msg)
+        return
+    seen[i] = None
+
+  threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+  for t in threads:
+    t.start()
+  for t in threads:
+    t.join()
+  assert seen == {0: None, 1: None, 2: None, 3: None}
+
+
 def test_host_noise_twin_matches_oracle_stream(lib):
   import oracle
   E = ft.ops.seeded_exp_rand(2, 3, 17, 33, 987654321987, "cpu")
