@@ -714,6 +714,40 @@ def test_config5_ea_sima_b8_h16_s8192_d64(gpu):
   assert (o16.float().cpu() - ref16.float()).abs().max().item() <= 1.2e-7  # two fp16 subnormal steps
 
 
+# ------------------------------------------------------------------ seeded random shapes
+
+def _random_shapes(n, seed=2024):
+  rng = np.random.RandomState(seed)
+  out = []
+  for _ in range(n):
+    sq = int(rng.choice([1, 2, 31, 33, 64, 65, 127, 129, 190, 257, 300]))
+    skv = sq + int(rng.choice([0, 0, 1, 40, 130]))
+    out.append((int(rng.randint(1, 3)), sq, skv, int(rng.randint(1, 6)), int(rng.choice([64, 128])), bool(rng.randint(0, 2)),
+                bool(rng.randint(0, 4) == 0), int(rng.randint(0, 1000))))
+  return out
+
+
+@pytest.mark.parametrize("B,Sq,Skv,H,D,causal,bf16,seed", _random_shapes(14))
+def test_random_shapes(gpu, B, Sq, Skv, H, D, causal, bf16, seed):
+  dtype = torch.bfloat16 if bf16 else torch.float16
+  g = torch.Generator().manual_seed(seed)
+  q = torch.randn(B, Sq, H, D, generator=g).to(dtype)
+  k = torch.randn(B, Skv, H, D, generator=g).to(dtype)
+  v = torch.randn(B, Skv, H, D, generator=g).to(dtype)
+  qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+  if causal:
+    ref_o, r1, r2 = oracle.roco_forward(q, k, v)
+  else:
+    p = torch.softmax((torch.matmul(q.transpose(1, 2), k.transpose(1, 2).transpose(-2, -1)) / np.sqrt(D)).float(), -1)
+    ref_o, r1, r2 = torch.matmul(p.to(dtype), v.transpose(1, 2)).transpose(1, 2), p.sum(2), (p * p).sum(2)
+  out, s1, s2 = ops.roco(qd, kd, vd, causal=causal)
+  # bf16: see test_bf16_small_ragged for the score bars
+  check_o(out, ref_o, tight=2e-2 if bf16 else 4e-3)
+  check_score(s1, r1, rel=8e-3 if bf16 else 2e-3); check_score(s2, r2, rel=1.6e-2 if bf16 else 4e-3)
+  idx = ops.topk(s1, max(1, Skv // 8))
+  assert oracle.topk_agreement(idx.cpu(), r1, max(1, Skv // 8), rtol=1e-2 if bf16 else 2e-3) == 0
+
+
 # ------------------------------------------------------------------ HIP graph capture
 
 def test_calls_can_be_captured_in_a_hip_graph(gpu):
