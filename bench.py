@@ -112,6 +112,34 @@ def per_config_table(dev, only=None, iters=100):
   return rows
 
 
+def mfma_probe(dev):
+  """What the matrix pipe alone sustains on this chip: an MFMA-only loop (ft_probe_mfma) on all-zero and on N(0,1)
+  fp16 operands.  The chip is power-limited, so the second figure, not the published peak, is the rate the
+  contractions of this workload could reach with nothing else running."""
+  import ctypes
+  import torch
+  from flashtensor_amd import _lib
+  lib = _lib.load()
+  cus = torch.cuda.get_device_properties(dev).multi_processor_count
+  sink = torch.zeros(4, dtype=torch.float32, device=dev)
+  clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+  stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+  out = {}
+  for name, ops_ in (("zeros", torch.zeros(32768, dtype=torch.float16, device=dev)),
+                     ("normal", torch.randn(32768, dtype=torch.float16, device=dev))):
+    def run(iters):
+      _lib.check(lib.ft_probe_mfma(ops_.data_ptr(), cus, iters, sink.data_ptr(), clocks.data_ptr(), stream))
+    run(20000)  # ramp
+    torch.cuda.synchronize()
+    iters = 200000
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(); run(iters); e1.record(); e1.synchronize()
+    ms = e0.elapsed_time(e1)
+    c = clocks.cpu().tolist()
+    out[name] = {"tflops": round(cus * 8 * iters * 4 * 32768 / ms / 1e9, 1), "shader_clock_mhz": round(100.0 * c[0] / max(1, c[1]))}
+  return out
+
+
 def cpu_baseline(B, S, H, D, heads):
   """The oracle's eager H2O forward on `heads` of the H heads (heads are independent), host cores."""
   import torch
@@ -207,6 +235,7 @@ def main():
       "kernels_us": {"attn_fwd_kernel": round(attn_us, 1), "colstats_kernel": round(step_us - attn_us, 1),
                      "step_events": round(step_us, 1)},
   }
+  result["mfma_probe"] = mfma_probe(dev)
   if not args.no_configs:
     result["per_config"] = per_config_table(dev, args.only, args.config_iters)
   if not args.no_cpu:

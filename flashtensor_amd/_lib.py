@@ -17,7 +17,7 @@ ABI_VERSION = 3
 # every symbol include/ft_abi.h declares
 EXPORTS = ("ft_abi_version", "ft_last_error", "ft_workspace_bytes", "ft_attn_fwd", "ft_attn_colstats_fwd",
            "ft_keyformer_fwd", "ft_attn_softcap_fwd", "ft_corm_fwd", "ft_avgpool1d", "ft_linattn_fwd", "ft_topk",
-           "ft_noise_exp_fill", "ft_noise_exp_fill_host", "ft_linattn_block_workspace_bytes", "ft_linattn_block_fwd")
+           "ft_noise_exp_fill", "ft_noise_exp_fill_host", "ft_linattn_block_workspace_bytes", "ft_linattn_block_fwd", "ft_probe_mfma")
 
 
 class FtStrides(ctypes.Structure):
@@ -96,6 +96,8 @@ def load():
   lib.ft_linattn_block_workspace_bytes.argtypes = [block_p, ctypes.c_int]
   lib.ft_linattn_block_fwd.restype = ctypes.c_int
   lib.ft_linattn_block_fwd.argtypes = [block_p, ctypes.c_int, ctypes.c_int, vp, ctypes.c_size_t, vp]
+  lib.ft_probe_mfma.restype = ctypes.c_int
+  lib.ft_probe_mfma.argtypes = [vp, ctypes.c_int32, ctypes.c_int32, f32p, vp, vp]
   if lib.ft_abi_version() != ABI_VERSION:
     raise ImportError(f"ABI version mismatch: library {lib.ft_abi_version()}, binding {ABI_VERSION}")
   _lib = lib

@@ -25,6 +25,7 @@ hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* 
 hipError_t launch_noise_fill(float* dst, int B, int H, int Sq, int Skv, uint64_t seed, hipStream_t s);
 hipError_t launch_avgpool1d(const float* src, int64_t rows, int S, int kernel, float* dst, hipStream_t s);
 hipError_t launch_group_mean(const float* src, int64_t groups, int group, int S, float* dst, hipStream_t s);
+hipError_t launch_mfma_probe(const void* operands, int workgroups, int iters, float* sink, long long* clocks, hipStream_t s);
 }  // namespace ft
 
 namespace {
@@ -451,6 +452,15 @@ int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx
   if (rows > 0x7fffffffLL) return fail(FT_EUNSUPPORTED, "too many rows");
   hipError_t e = ft::launch_topk(score, rows, S, k, idx, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "topk launch");
+  return FT_OK;
+}
+
+int ft_probe_mfma(const void* operands, int32_t workgroups, int32_t iters, float* sink, int64_t* clocks, void* stream) {
+  if (!operands || !sink) return fail(FT_EINVAL, "operands / sink pointer is null");
+  if (!aligned16(operands)) return fail(FT_EINVAL, "operands must be 16-byte aligned");
+  if (workgroups < 1 || workgroups > 65535 || iters < 1) return fail(FT_EINVAL, "bad probe size workgroups=%d iters=%d", workgroups, iters);
+  hipError_t e = ft::launch_mfma_probe(operands, workgroups, iters, sink, (long long*)clocks, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "mfma probe launch");
   return FT_OK;
 }
 

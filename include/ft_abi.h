@@ -157,6 +157,13 @@ int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx
 int ft_noise_exp_fill(float* dst, int32_t B, int32_t H, int32_t Sq, int32_t Skv, uint64_t seed, void* stream);
 int ft_noise_exp_fill_host(float* dst, int32_t B, int32_t H, int32_t Sq, int32_t Skv, uint64_t seed);
 
+/* Diagnostic, no counterpart in the reference: what the matrix pipe sustains on given operand values.
+ * `workgroups` workgroups of 8 waves each issue 4 * iters v_mfma_f32_32x32x16_f16 (32768 FLOP each) on fp16
+ * fragments read from `operands` (64 KiB, any values) and nothing else; time the launch with events on the
+ * stream.  clocks (optional, 2 x int64): shader-clock ticks and 100 MHz ticks one wave counted over its loop.
+ * The chip is power-limited, so the rate depends on the bit patterns of the operands.  sink: >= 4 bytes, unused. */
+int ft_probe_mfma(const void* operands, int32_t workgroups, int32_t iters, float* sink, int64_t* clocks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -158,6 +158,13 @@ def test_linear_block_argument_checks(lib):
   assert lib.ft_linattn_block_fwd(ctypes.byref(nul), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
 
 
+def test_probe_argument_checks(lib):
+  assert lib.ft_probe_mfma(None, 256, 10, 0x1000, None, None) == _lib.FT_EINVAL
+  assert lib.ft_probe_mfma(0x1008, 256, 10, 0x1000, None, None) == _lib.FT_EINVAL
+  assert lib.ft_probe_mfma(0x1000, 0, 10, 0x1000, None, None) == _lib.FT_EINVAL
+  assert lib.ft_probe_mfma(0x1000, 256, 0, 0x1000, None, None) == _lib.FT_EINVAL
+
+
 def test_last_error_is_per_thread(lib):
   import threading
   seen, barrier = {}, threading.Barrier(4)

@@ -790,6 +790,21 @@ def test_calls_can_be_captured_in_a_hip_graph(gpu):
       assert torch.equal(g, e)
 
 
+def test_mfma_probe_runs_and_reports_clocks(gpu):
+  import ctypes
+  from flashtensor_amd import _lib
+  lib = _lib.load()
+  operands = torch.randn(32768, dtype=torch.float16, device=gpu)
+  sink = torch.zeros(4, dtype=torch.float32, device=gpu)
+  clocks = torch.zeros(2, dtype=torch.int64, device=gpu)
+  _lib.check(lib.ft_probe_mfma(operands.data_ptr(), 64, 2000, sink.data_ptr(), clocks.data_ptr(),
+                               ctypes.c_void_p(torch.cuda.current_stream(gpu).cuda_stream)))
+  torch.cuda.synchronize()
+  shader, wall = clocks.cpu().tolist()
+  assert shader >= 2000 * 4 * 8 and wall > 0            # at least eight passes per MFMA... and the wall clock moved
+  assert 500 < 100.0 * shader / wall < 3000              # a shader clock in MHz
+
+
 # ------------------------------------------------------------------ command-line harness
 
 def test_cli_builds_and_runs_every_case(gpu, capsys):
