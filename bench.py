@@ -236,6 +236,7 @@ def main():
                      "step_events": round(step_us, 1)},
   }
   result["mfma_probe"] = mfma_probe(dev)
+  result["mfma_probe"]["attn_fwd_kernel_frac_of_normal"] = round(attn_tflops / result["mfma_probe"]["normal"]["tflops"], 4)
   if not args.no_configs:
     result["per_config"] = per_config_table(dev, args.only, args.config_iters)
   if not args.no_cpu:
