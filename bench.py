@@ -56,7 +56,11 @@ def per_config_table(dev, only=None, iters=100):
   def add(name, shape, fn, flops, nbytes):
     if only is not None and only not in name:
       return
-    us = event_time_us(fn, iters)
+    try:
+      us = event_time_us(fn, iters)
+    except Exception as e:  # a row that cannot run (hipBLASLt absent, say) is reported, the line is still printed
+      rows.append({"config": name, "shape": shape, "error": f"{type(e).__name__}: {e}"})
+      return
     tf, gb = flops / us / 1e6, nbytes / us / 1e3
     rows.append({"config": name, "shape": shape, "us": round(us, 1), "tflops": round(tf, 1),
                  "mfma_frac": round(tf / PEAK_MFMA_TFLOPS, 4), "gbs": round(gb, 1), "hbm_frac": round(gb / PEAK_HBM_GBS, 4)})
