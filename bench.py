@@ -239,8 +239,11 @@ def main():
       "kernels_us": {"attn_fwd_kernel": round(attn_us, 1), "colstats_kernel": round(step_us - attn_us, 1),
                      "step_events": round(step_us, 1)},
   }
-  result["mfma_probe"] = mfma_probe(dev)
-  result["mfma_probe"]["attn_fwd_kernel_frac_of_normal"] = round(attn_tflops / result["mfma_probe"]["normal"]["tflops"], 4)
+  try:
+    result["mfma_probe"] = mfma_probe(dev)
+    result["mfma_probe"]["attn_fwd_kernel_frac_of_normal"] = round(attn_tflops / result["mfma_probe"]["normal"]["tflops"], 4)
+  except Exception as e:  # diagnostic only: never costs the line
+    result["mfma_probe"] = {"error": f"{type(e).__name__}: {e}"}
   if not args.no_configs:
     result["per_config"] = per_config_table(dev, args.only, args.config_iters)
   if not args.no_cpu:
