@@ -12,7 +12,7 @@ FT_OK, FT_EINVAL, FT_EUNSUPPORTED, FT_ELAUNCH, FT_EWORKSPACE = 0, -1, -2, -3, -4
 FT_F16, FT_BF16, FT_F32 = 0, 1, 2
 FT_CAUSAL, FT_FAST_LOGITS = 1, 2
 FT_OP_ATTN, FT_OP_COLSTATS, FT_OP_KEYFORMER, FT_OP_EA, FT_OP_SIMA, FT_OP_CORM = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 # every symbol include/ft_abi.h declares
 EXPORTS = ("ft_abi_version", "ft_last_error", "ft_workspace_bytes", "ft_attn_fwd", "ft_attn_colstats_fwd",

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FT_ABI_VERSION 3
+#define FT_ABI_VERSION 4
 
 enum FtStatus {
   FT_OK = 0,

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(lib):
   assert declared == sorted(_lib.EXPORTS)
   for name in declared:
     assert getattr(lib, name) is not None
-  assert lib.ft_abi_version() == 3 == _lib.ABI_VERSION
+  assert lib.ft_abi_version() == 4 == _lib.ABI_VERSION
 
 
 def _args(**over):
