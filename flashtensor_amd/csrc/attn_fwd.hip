@@ -18,6 +18,7 @@
 #include "kernel_params.h"
 #include "noise.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace ft {
@@ -597,14 +598,15 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 // host-side launcher
 
 static int device_cu_count() {
-  static int cus[16] = {0};
+  static std::atomic<int> cus[16];  // zero-initialised; a racing first call stores the same value twice
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 256;
-  if (cus[dev] == 0) {
-    int n = 0;
-    cus[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  return cus[dev];
+  return n;
 }
 
 template <typename T, int D, bool CAUSAL, bool EMU, int KF>
