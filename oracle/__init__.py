@@ -16,5 +16,5 @@ from .cases import (  # noqa: F401
     ea_block_forward, sima_block_forward, prepare_block_inputs,
     prepare_inputs, prepare_exp_rand, heavy_hitters, roco_mean_var, chunked_over_heads,
 )
-from .noise import seeded_exp_rand, noise_u32, lowbias32  # noqa: F401
+from .noise import seeded_exp_rand, seeded_exp_rand_pairs, noise_u32, lowbias32  # noqa: F401
 from .metrics import loss, topk_agreement  # noqa: F401

@@ -64,3 +64,16 @@ def seeded_exp_rand(seed, B, H, Sq, Skv, row_offset=0):
       u = ((x >> np.uint32(9)).astype(np.float64) + 0.5) * 2.0 ** -23
       out[b, h] = (-np.log(u)).astype(np.float32)
   return torch.from_numpy(out)
+
+
+def seeded_exp_rand_pairs(seed, H_total, pairs, Sq, Skv):
+  """E for chosen (b, h) pairs of a problem with H_total heads, stacked as [1, len(pairs), Sq, Skv]: what
+  `seeded_exp_rand(seed, B, H_total, Sq, Skv)[b, h]` holds for each pair, without the other heads."""
+  import torch
+  out = np.empty((1, len(pairs), Sq, Skv), dtype=np.float32)
+  rows, cols = np.arange(Sq), np.arange(Skv)
+  for n, (b, h) in enumerate(pairs):
+    x = noise_u32(seed, b * H_total + h, rows, cols)
+    u = ((x >> np.uint32(9)).astype(np.float64) + 0.5) * 2.0 ** -23
+    out[0, n] = (-np.log(u)).astype(np.float32)
+  return torch.from_numpy(out)

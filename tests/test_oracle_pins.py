@@ -400,3 +400,76 @@ def test_attn2d_and_grouped_h2o_against_expanded_heads_and_brute_force():
   # unmasked variant: every key is visible to every row
   of, sf = oracle.attn_h2o2d_forward(q2, k2, v2, H, H, D, masked=False)
   assert abs(sf.sum().item() - H * S) < 1e-3 * S and (sf[:, -1] > 0.1).all()
+
+
+# ------------------------------------------------------------------ RoCo mean / variance epilogue, harness metrics
+
+def _mean_var_impls():
+  from flashtensor_amd import kernels
+  return [("oracle", oracle.roco_mean_var), ("product", kernels.RoCo.mean_var)]
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_roco_mean_var_zero_q_closed_form(which):
+  """q == 0: p_ij = 1/(i+1) for j <= i, else 0.  Over the S query rows key j then has
+  mean_j = (H_S - H_j) / S and population variance sum_{i>=j} (i+1)^-2 / S - mean_j^2; a variance that
+  forgets mean^2, divides by S - 1, or takes the mean over the visible rows only fails."""
+  name, fn = _mean_var_impls()[which]
+  S = 80
+  q, k, v = _inputs(S=S, D=64, seed=1)
+  _, s1, s2 = oracle.roco_forward(torch.zeros_like(q), k, v)
+  mean, var = fn(s1, s2, S)
+  inv = 1.0 / np.arange(1, S + 1)
+  ref_mean = np.cumsum(inv[::-1])[::-1] / S
+  ref_var = np.cumsum((inv ** 2)[::-1])[::-1] / S - ref_mean ** 2
+  assert np.abs(mean[0, 0].numpy() - ref_mean).max() < 1e-7, name
+  assert np.abs(var[0, 1].numpy() - ref_var).max() < 1e-7, name
+  # the wrong formulas are far outside that bar
+  assert np.abs(np.cumsum((inv ** 2)[::-1])[::-1] / S - ref_var).max() > 1e-3
+  assert np.abs((ref_var * S / (S - 1)) - ref_var).max() > 1e-5
+
+
+@pytest.mark.parametrize("which", [0, 1])
+@pytest.mark.parametrize("S,Skv", [(48, 48), (24, 56)])
+def test_roco_mean_var_against_numpy_on_brute_force_probs(which, S, Skv):
+  """mean / var over the query axis of the fp64 masked probability matrix (masked pairs are zeros, as in
+  probs.mean(2) / probs.var(2, unbiased=False) of the eager tensors of cases/kernels/roco.py:42-46)."""
+  name, fn = _mean_var_impls()[which]
+  q, k, v = _inputs(B=1, S=S, H=2, D=64, seed=9, kv_len=Skv)
+  _, s1, s2 = oracle.roco_forward(q, k, v)
+  mean, var = fn(s1, s2, S)
+  for h in range(2):
+    _, p = brute._probs(q.numpy(), k.numpy(), 0, h)
+    assert p.shape == (S, Skv)
+    np.testing.assert_allclose(mean[0, h].numpy(), p.mean(axis=0), rtol=2e-3, atol=1e-7, err_msg=name)
+    np.testing.assert_allclose(var[0, h].numpy(), p.var(axis=0), rtol=6e-3, atol=1e-7, err_msg=name)
+
+
+def _loss_impls():
+  from flashtensor_amd import utils
+  from oracle import metrics
+  return [("oracle", metrics.loss), ("product", utils.loss)]
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_loss_known_answers(which):
+  """python/asuka/utils.py:61-76 by hand: |d| = [0.5, 0, 1, 2], |ref| = [1, 2, 4, 0]."""
+  name, loss = _loss_impls()[which]
+  out = torch.tensor([[1.5, 2.0], [-3.0, 2.0]], dtype=torch.float16)
+  ref = torch.tensor([[1.0, 2.0], [-4.0, 0.0]], dtype=torch.float16)
+  r = loss(out, ref, remove_zero=True)       # the zero denominator becomes 1: rel = [0.5, 0, 0.25, 2]
+  assert r["remove_zero"] is True
+  assert r["abs_max"] == 2.0 and r["abs_mean"] == pytest.approx(0.875)
+  assert r["rel_max"] == 2.0 and r["rel_mean"] == pytest.approx(0.6875)
+  r = loss(out, ref)                          # kept: 2 / 0 = inf
+  assert r["remove_zero"] is False and r["abs_max"] == 2.0 and math.isinf(r["rel_max"]) and math.isinf(r["rel_mean"])
+  r = loss(out[:1], ref[:1])                  # no zero in the reference: rel = [0.5, 0]
+  assert r["rel_max"] == 0.5 and r["rel_mean"] == 0.25 and r["abs_mean"] == 0.25
+  assert not ref[1, 1].item() and ref.dtype == torch.float16   # the inputs are left as they were
+  # integer tensors: mismatch count and fraction
+  for dt in (torch.int32, torch.int64):
+    a = torch.tensor([1, 2, 3, 4, 5], dtype=dt)
+    b = torch.tensor([1, 0, 3, 0, 5], dtype=dt)
+    assert loss(a, b) == {"err_num": 2, "err": 0.4}, name
+  with pytest.raises(AssertionError):
+    loss(torch.zeros(2, 3), torch.zeros(3, 2))
