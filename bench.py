@@ -28,7 +28,13 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 ATTN_TRAFFIC_BYTES = 194.93e6
 
 
-def event_time_us(fn, iters, warmup=20):
+KERNEL_TIMING_ITERS = 300    # timed launches of the kernel-alone and step event loops, whatever --steps says
+KERNEL_TIMING_WARMUP = 100
+RAMP_SECONDS = 1.5           # untimed steps before the warm-up the caller asked for: clocks at their sustained level
+
+
+def event_time_us(fn, iters=KERNEL_TIMING_ITERS, warmup=KERNEL_TIMING_WARMUP):
+  """Average device time per call from events on torch's current stream (the stream the operators launch on)."""
   import torch
   for _ in range(warmup):
     fn()
@@ -41,6 +47,34 @@ def event_time_us(fn, iters, warmup=20):
   end.record()
   end.synchronize()
   return start.elapsed_time(end) * 1e3 / iters
+
+
+def ramp(fn, seconds=RAMP_SECONDS):
+  """Run fn back to back for about `seconds` of wall time (untimed); returns the time actually spent."""
+  import torch
+  t0 = time.perf_counter()
+  while time.perf_counter() - t0 < seconds:
+    for _ in range(50):
+      fn()
+    torch.cuda.synchronize()
+  return time.perf_counter() - t0
+
+
+def host_us_per_call(dev, calls=2000):
+  """Host-side cost of one operator call (argument checks, two allocations, the ctypes call, the launch):
+  wall time of un-synchronised calls on a problem small enough that the device never falls behind."""
+  import torch
+  from flashtensor_amd import ops
+  q, k, v = (torch.randn(1, 64, 1, 128, dtype=torch.float16, device=dev) for _ in range(3))
+  for _ in range(200):
+    ops.attn(q, k, v)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(calls):
+    ops.attn(q, k, v)
+  dt = time.perf_counter() - t0
+  torch.cuda.synchronize()
+  return dt / calls * 1e6
 
 
 def per_config_table(dev, only=None, iters=100):
@@ -57,7 +91,7 @@ def per_config_table(dev, only=None, iters=100):
     if only is not None and only not in name:
       return
     try:
-      us = event_time_us(fn, iters)
+      us = event_time_us(fn, iters, warmup=max(20, iters // 4))
     except Exception as e:  # a row that cannot run (hipBLASLt absent, say) is reported, the line is still printed
       rows.append({"config": name, "shape": shape, "error": f"{type(e).__name__}: {e}"})
       return
@@ -117,13 +151,13 @@ def per_config_table(dev, only=None, iters=100):
 
 
 def mfma_probe(dev):
-  """What the matrix pipe alone sustains on this chip: an MFMA-only loop (ft_probe_mfma) on all-zero and on N(0,1)
-  fp16 operands.  The chip is power-limited, so the second figure, not the published peak, is the rate the
-  contractions of this workload could reach with nothing else running."""
+  """What the matrix pipe alone sustains on this chip: an MFMA-only loop (ft_diag_probe_mfma of the diagnostics
+  library, include/ft_diag.h) on all-zero and on N(0,1) fp16 operands.  The chip is power-limited, so the second
+  figure, not the published peak, is the rate the contractions of this workload could reach with nothing else running."""
   import ctypes
   import torch
   from flashtensor_amd import _lib
-  lib = _lib.load()
+  diag = _lib.load_diag()
   cus = torch.cuda.get_device_properties(dev).multi_processor_count
   sink = torch.zeros(4, dtype=torch.float32, device=dev)
   clocks = torch.zeros(2, dtype=torch.int64, device=dev)
@@ -132,7 +166,8 @@ def mfma_probe(dev):
   for name, ops_ in (("zeros", torch.zeros(32768, dtype=torch.float16, device=dev)),
                      ("normal", torch.randn(32768, dtype=torch.float16, device=dev))):
     def run(iters):
-      _lib.check(lib.ft_probe_mfma(ops_.data_ptr(), cus, iters, sink.data_ptr(), clocks.data_ptr(), stream))
+      if diag.ft_diag_probe_mfma(ops_.data_ptr(), ops_.numel() * 2, cus, iters, sink.data_ptr(), clocks.data_ptr(), stream) != 0:
+        raise RuntimeError(diag.ft_diag_last_error().decode())
     run(20000)  # ramp
     torch.cuda.synchronize()
     iters = 200000
@@ -163,7 +198,7 @@ def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
   ap.add_argument("--steps", type=int, default=500)
-  ap.add_argument("--warmup", type=int, default=200)
+  ap.add_argument("--warmup", type=int, default=100)
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
   ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
   ap.add_argument("--cpu-heads", type=int, default=4)
@@ -178,7 +213,7 @@ def main():
 
   import torch
   from flashtensor_amd import _lib, ops
-  _lib.load()  # the HIP library is the only execution path
+  _lib.ffi()  # the HIP library (through its pybind11 module) is the only execution path
   if not torch.cuda.is_available():
     sys.exit("bench.py: no GPU visible")
   dev = torch.device("cuda:0")
@@ -201,6 +236,7 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
+  ramp_s = ramp(step)  # untimed: a short run would otherwise be timed while the clocks are still settling
   for _ in range(args.warmup):
     step()
   torch.cuda.synchronize()
@@ -210,10 +246,12 @@ def main():
   torch.cuda.synchronize()
   dt = (time.perf_counter() - t0) / args.steps
 
-  # dominant kernel: the attention forward with its normaliser output, events on the launch stream
-  attn_us = event_time_us(lambda: ops.attn(q, k, v, return_lse=True), max(10, args.steps))
-  step_us = event_time_us(step, max(10, args.steps))
+  # dominant kernel: the attention forward with its normaliser output, events on the launch stream; a fixed
+  # number of launches, independent of --steps
+  attn_us = event_time_us(lambda: ops.attn(q, k, v, return_lse=True))
+  step_us = event_time_us(step)
   attn_tflops = flops / attn_us / 1e6
+  host_us = host_us_per_call(dev)
 
   result = {
       "metric": "fused attn+score (H2O) algorithmic TFLOP/s at S=4096, 1 GPU",
@@ -223,6 +261,8 @@ def main():
       "steps": args.steps,
       "warmup": args.warmup,
       "ms_per_step": round(dt * 1e3, 5),
+      "ramp_s": round(ramp_s, 2),
+      "host_us_per_call": round(host_us, 1),
       "us_per_step": round(dt * 1e6, 1),
       "higher_is_better": True,
       "scaling": "weak",
@@ -235,7 +275,8 @@ def main():
       "algorithmic_gbs": round(alg_bytes / dt / 1e9, 1),
       "roofline": {"bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(attn_tflops, 1), "peak": PEAK_MFMA_TFLOPS,
                    "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_MFMA_TFLOPS, 4), "traffic": ATTN_TRAFFIC_BYTES,
-                   "us_per_launch": round(attn_us, 1), "algorithmic_flop_per_launch": flops},
+                   "us_per_launch": round(attn_us, 1), "algorithmic_flop_per_launch": flops,
+                   "timed_launches": KERNEL_TIMING_ITERS},
       "kernels_us": {"attn_fwd_kernel": round(attn_us, 1), "colstats_kernel": round(step_us - attn_us, 1),
                      "step_events": round(step_us, 1)},
   }

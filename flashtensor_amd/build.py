@@ -14,8 +14,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libflashtensor_hip.so")
+DIAG_LIB_PATH = os.path.join(HERE, "libflashtensor_diag.so")  # include/ft_diag.h: probes for the benchmark, not product
 SOURCES = ["abi.hip", "attn_fwd.hip", "colstats.hip", "linattn.hip", "aux.hip", "linblock.hip"]
-HEADERS = ["device_common.hpp", "kernel_params.h", "noise.h", os.path.join("..", "..", "include", "ft_abi.h")]
+DIAG_SOURCES = ["diag.hip"]
+FFI_SOURCE = "ffi_kernels.cpp"  # pybind11 module ft_ffi over the C ABI (plain C++: no device code, no torch headers)
+HEADERS = ["device_common.hpp", "kernel_params.h", "noise.h", os.path.join("..", "..", "include", "ft_abi.h"),
+           os.path.join("..", "..", "include", "ft_diag.h")]
 # packed fp32 VALU ops are disabled on purpose: some forms have produced wrong results on this hardware
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
@@ -46,18 +50,49 @@ def _compile(src, force):
   return obj, res.stderr
 
 
-def build(force=False, verbose=True):
-  os.makedirs(OBJ_DIR, exist_ok=True)
-  with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-    results = list(ex.map(lambda s: _compile(s, force), SOURCES))
-  objs = [o for o, _ in results]
-  if force or _stale(LIB_PATH, objs):
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+def _link(lib_path, objs, force):
+  if force or _stale(lib_path, objs):
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
       raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+
+
+def ffi_path():
+  import sysconfig
+  return os.path.join(HERE, "ft_ffi" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def _build_ffi(force):
+  """g++ on csrc/ffi_kernels.cpp against pybind11 and the Python headers, linked to libflashtensor_hip.so
+  (found next to the module through an $ORIGIN run path)."""
+  import sysconfig
+  import pybind11
+  out = ffi_path()
+  src = os.path.join(CSRC, FFI_SOURCE)
+  deps = [src, os.path.join(HERE, "..", "include", "ft_abi.h"), LIB_PATH]
+  if not force and not _stale(out, deps):
+    return out
+  cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+         "-I" + pybind11.get_include(), "-I" + sysconfig.get_paths()["include"], src, "-o", out,
+         "-L" + HERE, "-lflashtensor_hip", "-Wl,-rpath,$ORIGIN"]
+  res = subprocess.run(cmd, capture_output=True, text=True)
+  if res.returncode != 0:
+    raise RuntimeError(f"building ft_ffi failed:\n{res.stdout}\n{res.stderr}")
+  return out
+
+
+def build(force=False, verbose=True):
+  os.makedirs(OBJ_DIR, exist_ok=True)
+  sources = SOURCES + DIAG_SOURCES
+  with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources))) as ex:
+    results = list(ex.map(lambda s: _compile(s, force), sources))
+  objs = [o for o, _ in results]
+  _link(LIB_PATH, objs[:len(SOURCES)], force)
+  _link(DIAG_LIB_PATH, objs[len(SOURCES):], force)
+  ffi = _build_ffi(force)
   if verbose:
-    print(f"built {LIB_PATH}")
+    print(f"built {LIB_PATH}, {DIAG_LIB_PATH} and {ffi}")
   return LIB_PATH
 
 

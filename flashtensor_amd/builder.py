@@ -31,7 +31,7 @@ class HipBuilder(Builder):
     self.hyper = hyper
 
   def build_callable(self) -> Callable[..., Any]:
-    _lib.load()  # fail here, not at the first call, when the HIP library is missing
+    _lib.ffi()  # fail here, not at the first call, when the HIP library is missing
     model = get_model(self.kernel, **self.hyper)
     if not self.check_before_run:
       return model.forward

@@ -8,6 +8,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 
@@ -25,7 +26,6 @@ hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* 
 hipError_t launch_noise_fill(float* dst, int B, int H, int Sq, int Skv, uint64_t seed, hipStream_t s);
 hipError_t launch_avgpool1d(const float* src, int64_t rows, int S, int kernel, float* dst, hipStream_t s);
 hipError_t launch_group_mean(const float* src, int64_t groups, int group, int S, float* dst, hipStream_t s);
-hipError_t launch_mfma_probe(const void* operands, int workgroups, int iters, float* sink, long long* clocks, hipStream_t s);
 }  // namespace ft
 
 namespace {
@@ -127,10 +127,14 @@ float tuned_logit_multiplier(int D, bool bf16) {
 // fp16 h whose quotient is at least 2.5e-3 in magnitude, and is within 2e-6 * 8 of it below (checked here over
 // all 65536 inputs on first use; a logit that small moves a probability by 2e-6 relative).  D = 64 needs no
 // constants: h / 8 is exact.
-bool packed_logit_constants(uint32_t* hi2, uint32_t* lo2) {
-  static int verified = 0;  // 0 unknown, 1 good, -1 bad
-  const _Float16 hi = (_Float16)0.70751953125f, lo = (_Float16)-0.0004127025604248047f;
-  if (verified == 0) {
+struct PackedLogitConstants {
+  uint32_t hi2, lo2;  // the constant in both halves of a 32-bit word
+  bool good;          // the exhaustive check passed
+};
+const PackedLogitConstants& packed_logit_constants() {
+  // a function-local static is initialised exactly once per process, by whichever thread gets here first
+  static const PackedLogitConstants consts = [] {
+    const _Float16 hi = (_Float16)0.70751953125f, lo = (_Float16)-0.0004127025604248047f;
     bool ok = true;
     const float c = (float)std::sqrt(128.0);
     for (uint32_t bits = 0; bits < 65536 && ok; ++bits) {
@@ -141,12 +145,10 @@ bool packed_logit_constants(uint32_t* hi2, uint32_t* lo2) {
       const double got = (double)(float)(_Float16)((double)x * (double)(float)hi + cterm) / 8.0;
       if (got != want && (std::fabs(want) >= 2.5e-3 || std::fabs(got - want) > 2e-6)) ok = false;
     }
-    verified = ok ? 1 : -1;
-  }
-  const uint16_t hb = float_to_half_bits((float)hi), lb = float_to_half_bits((float)lo);
-  *hi2 = (uint32_t)hb | ((uint32_t)hb << 16);
-  *lo2 = (uint32_t)lb | ((uint32_t)lb << 16);
-  return verified == 1;
+    const uint16_t hb = float_to_half_bits((float)hi), lb = float_to_half_bits((float)lo);
+    return PackedLogitConstants{(uint32_t)hb | ((uint32_t)hb << 16), (uint32_t)lb | ((uint32_t)lb << 16), ok};
+  }();
+  return consts;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -161,10 +163,7 @@ int validate_attn(const FtAttnArgs* a, bool need_v_o) {
   if (a->Hkv < 0 || (a->Hkv > 0 && (a->Hkv > a->H || a->H % a->Hkv != 0)))
     return fail(FT_EINVAL, "bad head grouping H=%d Hkv=%d (H must be a multiple of Hkv)", a->H, a->Hkv);
   if (a->D != 64 && a->D != 128) return fail(FT_EUNSUPPORTED, "head_dim %d not supported (64 or 128)", a->D);
-  {
-    uint32_t hi2, lo2;
-    if (!packed_logit_constants(&hi2, &lo2)) return fail(FT_EUNSUPPORTED, "internal: packed logit constants failed their exhaustive check");
-  }
+  if (!packed_logit_constants().good) return fail(FT_EUNSUPPORTED, "internal: packed logit constants failed their exhaustive check");
   if (a->dtype != FT_F16 && a->dtype != FT_BF16) return fail(FT_EUNSUPPORTED, "dtype %d not supported (f16 or bf16)", a->dtype);
   if ((a->flags & FT_CAUSAL) && a->Skv < a->Sq)
     return fail(FT_EINVAL, "causal mask needs Skv >= Sq (got Sq=%d Skv=%d): rows without a visible key are undefined", a->Sq, a->Skv);
@@ -208,7 +207,8 @@ ft::AttnKernelParams attn_params(const FtAttnArgs* a, bool emu) {
                     : (float)(1.4426950408889634 / std::sqrt((double)a->D));
   p.inv_tau = 1.f;
   p.group = group_of(a);
-  packed_logit_constants(&p.pk_hi2, &p.pk_lo2);
+  p.pk_hi2 = packed_logit_constants().hi2;
+  p.pk_lo2 = packed_logit_constants().lo2;
   return p;
 }
 
@@ -231,7 +231,8 @@ ft::ColstatsKernelParams col_params(const FtAttnArgs* a, bool emu, const float* 
                     : (float)(1.4426950408889634 / std::sqrt((double)a->D));
   p.inv_tau = 1.f;
   p.group = group_of(a);
-  packed_logit_constants(&p.pk_hi2, &p.pk_lo2);
+  p.pk_hi2 = packed_logit_constants().hi2;
+  p.pk_lo2 = packed_logit_constants().lo2;
   return p;
 }
 
@@ -239,6 +240,39 @@ size_t lse_bytes(const FtAttnArgs* a) { return (size_t)a->B * a->H * a->Sq * siz
 // grouped queries: the per-query-head column sums live in the workspace before their group mean is taken
 size_t colstats_bytes(const FtAttnArgs* a) {
   return lse_bytes(a) + (group_of(a) > 1 ? (size_t)a->B * a->H * a->Skv * sizeof(float) : 0);
+}
+
+
+int validate_colstats(const FtAttnArgs* a, const float* colsum, const float* colsumsq) {
+  if (int rc = validate_attn(a, true)) return rc;
+  if (!colsum) return fail(FT_EINVAL, "colsum pointer is null");
+  const int group = group_of(a);
+  if (group > 1 && colsumsq) return fail(FT_EUNSUPPORTED, "sum of squares is not defined per query head under grouped queries");
+  if (group > 1 && (int64_t)a->B * a->Hkv > 65535) return fail(FT_EUNSUPPORTED, "too many k/v heads for the group mean");
+  return FT_OK;
+}
+
+// attention pass (writes the row normalisers to the scratch), column pass, group mean when grouped; `ws` holds
+// colstats_bytes(a) bytes.  Every scratch element that is read has been written earlier in the same call.
+int run_colstats(const FtAttnArgs* a, float* colsum, float* colsumsq, void* ws, void* stream) {
+  const int group = group_of(a);
+  const bool emu = !(a->flags & FT_FAST_LOGITS);
+  const bool causal = a->flags & FT_CAUSAL;
+  float* lse = static_cast<float*>(ws);
+  float* per_head = group > 1 ? lse + (size_t)a->B * a->H * a->Sq : colsum;
+  ft::AttnKernelParams p = attn_params(a, emu);
+  p.lse = lse;
+  hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, causal, emu, ft::kKfNone, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "attn_fwd launch");
+  ft::ColstatsKernelParams c = col_params(a, emu, lse, per_head, colsumsq);
+  e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, colsumsq ? ft::kStatSumSq : ft::kStatSum,
+                          (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "colstats launch");
+  if (group > 1) {
+    e = ft::launch_group_mean(per_head, (int64_t)a->B * a->Hkv, group, a->Skv, colsum, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "group mean launch");
+  }
+  return FT_OK;
 }
 
 }  // namespace
@@ -279,32 +313,12 @@ int ft_attn_fwd(const FtAttnArgs* a, float* lse, void* stream) {
 
 int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, void* workspace, size_t workspace_bytes,
                          void* stream) {
-  if (int rc = validate_attn(a, true)) return rc;
-  if (!colsum) return fail(FT_EINVAL, "colsum pointer is null");
-  const int group = group_of(a);
-  if (group > 1 && colsumsq) return fail(FT_EUNSUPPORTED, "sum of squares is not defined per query head under grouped queries");
+  if (int rc = validate_colstats(a, colsum, colsumsq)) return rc;
   const size_t need = colstats_bytes(a);
   if (!workspace || workspace_bytes < need)
     return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
   if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(FT_EINVAL, "workspace must be 4-byte aligned");
-  const bool emu = !(a->flags & FT_FAST_LOGITS);
-  const bool causal = a->flags & FT_CAUSAL;
-  float* lse = static_cast<float*>(workspace);
-  float* per_head = group > 1 ? lse + (size_t)a->B * a->H * a->Sq : colsum;
-  ft::AttnKernelParams p = attn_params(a, emu);
-  p.lse = lse;
-  hipError_t e = ft::launch_attn_fwd(p, a->D, a->dtype == FT_BF16, causal, emu, ft::kKfNone, (hipStream_t)stream);
-  if (e != hipSuccess) return hip_fail(e, "attn_fwd launch");
-  ft::ColstatsKernelParams c = col_params(a, emu, lse, per_head, colsumsq);
-  e = ft::launch_colstats(c, a->D, a->dtype == FT_BF16, causal, emu, colsumsq ? ft::kStatSumSq : ft::kStatSum,
-                          (hipStream_t)stream);
-  if (e != hipSuccess) return hip_fail(e, "colstats launch");
-  if (group > 1) {
-    if ((int64_t)a->B * a->Hkv > 65535) return fail(FT_EUNSUPPORTED, "too many k/v heads for the group mean");
-    e = ft::launch_group_mean(per_head, (int64_t)a->B * a->Hkv, group, a->Skv, colsum, (hipStream_t)stream);
-    if (e != hipSuccess) return hip_fail(e, "group mean launch");
-  }
-  return FT_OK;
+  return run_colstats(a, colsum, colsumsq, workspace, stream);
 }
 
 int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float* kf_score, void* workspace,
@@ -452,15 +466,6 @@ int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx
   if (rows > 0x7fffffffLL) return fail(FT_EUNSUPPORTED, "too many rows");
   hipError_t e = ft::launch_topk(score, rows, S, k, idx, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "topk launch");
-  return FT_OK;
-}
-
-int ft_probe_mfma(const void* operands, int32_t workgroups, int32_t iters, float* sink, int64_t* clocks, void* stream) {
-  if (!operands || !sink) return fail(FT_EINVAL, "operands / sink pointer is null");
-  if (!aligned16(operands)) return fail(FT_EINVAL, "operands must be 16-byte aligned");
-  if (workgroups < 1 || workgroups > 65535 || iters < 1) return fail(FT_EINVAL, "bad probe size workgroups=%d iters=%d", workgroups, iters);
-  hipError_t e = ft::launch_mfma_probe(operands, workgroups, iters, sink, (long long*)clocks, (hipStream_t)stream);
-  if (e != hipSuccess) return hip_fail(e, "mfma probe launch");
   return FT_OK;
 }
 

@@ -159,45 +159,4 @@ hipError_t launch_group_mean(const float* src, int64_t groups, int group, int S,
   return hipGetLastError();
 }
 
-// Diagnostic: the rate the matrix pipe sustains on the caller's operands.  Every wave of a 512-thread workgroup
-// keeps four independent 32x32 accumulators and issues nothing but v_mfma_f32_32x32x16_f16 on fragments read
-// from `operands` (4096 x 16 bytes); clocks[0..1] receive one wave's shader-clock and 100 MHz wall-clock ticks
-// over the loop.  The chip is power-limited: the answer depends on the bit patterns (all-zero operands run at
-// the full clock, N(0,1) values at about two thirds of it).
-__global__ void __launch_bounds__(512) mfma_probe_kernel(const uint4v* __restrict__ operands, int iters, float* __restrict__ sink,
-                                                         long long* __restrict__ clocks) {
-  half8 a[4], b[4];
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    a[u] = __builtin_bit_cast(half8, operands[(threadIdx.x + 512 * u) & 4095]);
-    b[u] = __builtin_bit_cast(half8, operands[(threadIdx.x + 512 * u + 2048) & 4095]);
-  }
-  float16v c[4];
-#pragma unroll
-  for (int u = 0; u < 4; ++u)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) c[u][r] = 0.f;
-  const long long t0 = clock64(), w0 = wall_clock64();
-  for (int it = 0; it < iters; ++it) {
-#pragma unroll
-    for (int u = 0; u < 4; ++u) c[u] = F16::mfma(a[u], b[(u + 1) & 3], c[u]);
-  }
-  const long long t1 = clock64(), w1 = wall_clock64();
-  float acc = 0.f;
-#pragma unroll
-  for (int u = 0; u < 4; ++u)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc += c[u][r];
-  if (acc == 12345.678f) sink[0] = acc;  // keeps the loop alive
-  if (threadIdx.x == 0 && blockIdx.x == 0 && clocks) {
-    clocks[0] = t1 - t0;
-    clocks[1] = w1 - w0;
-  }
-}
-
-hipError_t launch_mfma_probe(const void* operands, int workgroups, int iters, float* sink, long long* clocks, hipStream_t s) {
-  hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)workgroups), dim3(512), 0, s, (const uint4v*)operands, iters, sink, clocks);
-  return hipGetLastError();
-}
-
 }  // namespace ft

@@ -3,20 +3,24 @@
 Call convention of the reference's emitted kernel wrapper (lib/Translate/to_triton.cpp:540-609): positional
 torch tensors in, results allocated with torch.empty on the device of the first argument and returned
 (a tuple when there are several), launch on the current stream, no synchronisation.  Torch is used for
-device memory and the stream handle only; all arithmetic happens in libflashtensor_hip.
+device memory and the stream handle only; all arithmetic happens in libflashtensor_hip, reached through the
+pybind11 module ft_ffi (csrc/ffi_kernels.cpp, the counterpart of the reference's ffi/ layer): bad arguments
+raise ValueError, everything else RuntimeError, as std::invalid_argument / std::runtime_error do there
+(ffi/passes.cpp:81-83).
 """
-import ctypes
-
 import torch
 
 from . import _lib
-from ._lib import FtAttnArgs, FtNoise, FtStrides
 
 _DTYPES = {torch.float16: _lib.FT_F16, torch.bfloat16: _lib.FT_BF16}
 
 
+def _k():
+  return _lib.ffi().kernels
+
+
 def _stream(t):
-  return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+  return torch.cuda.current_stream(t.device).cuda_stream
 
 
 def _check_qkv(q, k, v):
@@ -40,17 +44,17 @@ def _check_qkv(q, k, v):
 
 
 def _dense_last(t):
-  return t if t.stride(-1) == 1 else t.contiguous()
-
-
-def _strides(t):
-  return FtStrides(t.stride(0), t.stride(1), t.stride(2))
+  """The kernels read rows of contiguous elements; a tensor whose last axis is strided is refused (as the C
+  ABI refuses it) rather than copied behind the caller's back."""
+  if t.stride(-1) != 1 and t.shape[-1] != 1:
+    raise ValueError(f"need a contiguous last axis but got strides {tuple(t.stride())} for shape {tuple(t.shape)}")
+  return t
 
 
 def _args(q, k, v, o, flags):
   B, Sq, H, D = q.shape
-  return FtAttnArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _strides(q), _strides(k), _strides(v),
-                    _strides(o), B, H, Sq, k.shape[1], D, _DTYPES[q.dtype], flags, k.shape[2])
+  return _k().AttnArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), q.stride()[:3], k.stride()[:3], v.stride()[:3],
+                       o.stride()[:3], B, H, Sq, k.shape[1], D, _DTYPES[q.dtype], flags, k.shape[2])
 
 
 def _flags(causal, fast_logits):
@@ -66,27 +70,24 @@ def attn(q, k, v, causal=True, fast_logits=False, return_lse=False):
   """Attn.forward (cases/kernels/attn.py:18-34): q [B,S,H,D], k,v [B,Skv,Hkv,D] -> out [B,Sq,H,D].  With
   Hkv < H query head h attends to k/v head h // (H // Hkv), the grouping of cases/attn.py:29-31."""
   q, k, v = _prep(q, k, v)
-  lib = _lib.load()
   out = torch.empty_like(q, memory_format=torch.contiguous_format)
   lse = torch.empty(q.shape[0], q.shape[2], q.shape[1], dtype=torch.float32, device=q.device) if return_lse else None
-  a = _args(q, k, v, out, _flags(causal, fast_logits))
-  _lib.check(lib.ft_attn_fwd(ctypes.byref(a), lse.data_ptr() if return_lse else None, _stream(q)))
+  _k().attn_fwd(_args(q, k, v, out, _flags(causal, fast_logits)), lse.data_ptr() if return_lse else 0, _stream(q))
   return (out, lse) if return_lse else out
 
 
 def _colstats(q, k, v, want_sq, causal, fast_logits):
   q, k, v = _prep(q, k, v)
-  lib = _lib.load()
+  ffi = _k()
   B, Sq, H, D = q.shape
   Skv = k.shape[1]
   out = torch.empty_like(q, memory_format=torch.contiguous_format)
   s1 = torch.empty(B, k.shape[2], Skv, dtype=torch.float32, device=q.device)  # per k/v head (group mean when grouped)
   s2 = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device) if want_sq else None
   a = _args(q, k, v, out, _flags(causal, fast_logits))
-  nbytes = lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a))
+  nbytes = ffi.workspace_bytes(_lib.FT_OP_COLSTATS, a)
   ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-  _lib.check(lib.ft_attn_colstats_fwd(ctypes.byref(a), s1.data_ptr(), s2.data_ptr() if want_sq else None,
-                                      ws.data_ptr(), nbytes, _stream(q)))
+  ffi.attn_colstats_fwd(a, s1.data_ptr(), s2.data_ptr() if want_sq else 0, ws.data_ptr(), nbytes, _stream(q))
   return (out, s1, s2) if want_sq else (out, s1)
 
 
@@ -105,24 +106,23 @@ def keyformer(q, k, v, exp_rand=None, tau=1.5, seed=0, causal=True, fast_logits=
   """KeyFormer.forward (cases/kernels/kf.py:19-42) -> (out, kf_score [B,H,Skv] fp32).
   exp_rand [B,H,Sq,Skv] fp32 is the reference's noise input; None draws it in-kernel from `seed`."""
   q, k, v = _prep(q, k, v)
-  lib = _lib.load()
+  ffi = _k()
   B, Sq, H, D = q.shape
   Skv = k.shape[1]
-  noise = FtNoise(None, 0, 0, 0, int(seed) & 0xFFFFFFFFFFFFFFFF)
+  noise = ffi.Noise(0, 0, 0, 0, int(seed) & 0xFFFFFFFFFFFFFFFF)
   if exp_rand is not None:
     if tuple(exp_rand.shape) != (B, H, Sq, Skv):
       raise RuntimeError(f"arg 3 need shape {(B, H, Sq, Skv)} but got {tuple(exp_rand.shape)}")
     if exp_rand.dtype != torch.float32 or exp_rand.device != q.device:
       raise RuntimeError(f"arg 3 need dtype torch.float32 on {q.device} but got {exp_rand.dtype} on {exp_rand.device}")
     exp_rand = _dense_last(exp_rand)
-    noise = FtNoise(exp_rand.data_ptr(), exp_rand.stride(0), exp_rand.stride(1), exp_rand.stride(2), 0)
+    noise = ffi.Noise(exp_rand.data_ptr(), exp_rand.stride(0), exp_rand.stride(1), exp_rand.stride(2), 0)
   out = torch.empty_like(q, memory_format=torch.contiguous_format)
   score = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device)
   a = _args(q, k, v, out, _flags(causal, fast_logits))
-  nbytes = lib.ft_workspace_bytes(_lib.FT_OP_KEYFORMER, ctypes.byref(a))
+  nbytes = ffi.workspace_bytes(_lib.FT_OP_KEYFORMER, a)
   ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-  _lib.check(lib.ft_keyformer_fwd(ctypes.byref(a), ctypes.byref(noise), float(tau), score.data_ptr(), ws.data_ptr(),
-                                  nbytes, _stream(q)))
+  ffi.keyformer_fwd(a, noise, float(tau), score.data_ptr(), ws.data_ptr(), nbytes, _stream(q))
   return out, score
 
 
@@ -130,10 +130,9 @@ def snapkv(q, k, v, kernel_size=5, causal=True, fast_logits=False):
   """SnapKV.forward (cases/kernels/snapkv.py:19-43) -> (out, snapkv_score [B,H,Skv] fp32): the H2O column
   sums smoothed by a stride-1 average pool of odd width `kernel_size` over the key axis."""
   out, score = _colstats(q, k, v, False, causal, fast_logits)
-  lib = _lib.load()
   B, H, Skv = score.shape
   pooled = torch.empty_like(score)
-  _lib.check(lib.ft_avgpool1d(score.data_ptr(), B * H, Skv, int(kernel_size), pooled.data_ptr(), _stream(q)))
+  _k().avgpool1d(score.data_ptr(), B * H, Skv, int(kernel_size), pooled.data_ptr(), _stream(q))
   return out, pooled
 
 
@@ -142,10 +141,10 @@ def corm(q, k, v, corm_mask=None, causal=True, fast_logits=False, return_margin=
   query row gives it a probability >= corm_mask[i, j].  corm_mask [Sq,Skv] fp32 is the reference's input;
   None applies its prepare() recipe 1 / (i + 1) (corm.py:47-49) without reading a tensor."""
   q, k, v = _prep(q, k, v)
-  lib = _lib.load()
+  ffi = _k()
   B, Sq, H, D = q.shape
   Skv = k.shape[1]
-  mask_ptr, mask_stride = None, 0
+  mask_ptr, mask_stride = 0, 0
   if corm_mask is not None:
     if tuple(corm_mask.shape) != (Sq, Skv):
       raise RuntimeError(f"arg 3 need shape {(Sq, Skv)} but got {tuple(corm_mask.shape)}")
@@ -157,10 +156,10 @@ def corm(q, k, v, corm_mask=None, causal=True, fast_logits=False, return_margin=
   keep = torch.empty(B, H, Skv, dtype=torch.uint8, device=q.device)
   margin = torch.empty(B, H, Skv, dtype=torch.float32, device=q.device) if return_margin else None
   a = _args(q, k, v, out, _flags(causal, fast_logits))
-  nbytes = lib.ft_workspace_bytes(_lib.FT_OP_CORM, ctypes.byref(a))
+  nbytes = ffi.workspace_bytes(_lib.FT_OP_CORM, a)
   ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-  _lib.check(lib.ft_corm_fwd(ctypes.byref(a), mask_ptr, mask_stride, keep.data_ptr(),
-                             margin.data_ptr() if return_margin else None, ws.data_ptr(), nbytes, _stream(q)))
+  ffi.corm_fwd(a, mask_ptr, mask_stride, keep.data_ptr(), margin.data_ptr() if return_margin else 0, ws.data_ptr(), nbytes,
+               _stream(q))
   keep = keep.view(torch.bool)
   return (out, keep, margin) if return_margin else (out, keep)
 
@@ -168,27 +167,27 @@ def corm(q, k, v, corm_mask=None, causal=True, fast_logits=False, return_margin=
 def gemma2(q, k, v, softcap=50.0, causal=True, fast_logits=False):
   """Gemma2.forward (cases/kernels/gemma2.py:19-39): attention with logits softcap * tanh(logit / softcap)."""
   q, k, v = _prep(q, k, v)
-  lib = _lib.load()
   out = torch.empty_like(q, memory_format=torch.contiguous_format)
-  a = _args(q, k, v, out, _flags(causal, fast_logits))
-  _lib.check(lib.ft_attn_softcap_fwd(ctypes.byref(a), float(softcap), None, _stream(q)))
+  _k().attn_softcap_fwd(_args(q, k, v, out, _flags(causal, fast_logits)), float(softcap), 0, _stream(q))
   return out
 
 
 def _linattn(q, k, v, kind, normalize_q, out_dtype):
   q, k, v = _prep(q, k, v)
   if q.shape[3] == 32:  # head_dim 32 runs as pairs of adjacent heads: heads must lie 32 elements apart
-    q, k, v = (t if t.stride(2) == 32 else t.contiguous() for t in (q, k, v))
-  lib = _lib.load()
+    for i, t in enumerate((q, k, v)):
+      if t.stride(2) != 32:
+        raise ValueError(f"arg {i} with head_dim 32 need heads stored 32 elements apart but got head stride {t.stride(2)}")
+  ffi = _k()
   out_dtype = out_dtype or q.dtype
   if out_dtype not in (torch.float16, torch.float32):
     raise RuntimeError(f"out_dtype need float16 or float32 but got {out_dtype}")
   out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
   a = _args(q, k, v, out, 0)
-  nbytes = lib.ft_workspace_bytes(kind, ctypes.byref(a))
+  nbytes = ffi.workspace_bytes(kind, a)
   ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-  _lib.check(lib.ft_linattn_fwd(ctypes.byref(a), kind, int(bool(normalize_q)),
-                                _lib.FT_F32 if out_dtype == torch.float32 else _lib.FT_F16, ws.data_ptr(), nbytes, _stream(q)))
+  ffi.linattn_fwd(a, kind, int(bool(normalize_q)), _lib.FT_F32 if out_dtype == torch.float32 else _lib.FT_F16, ws.data_ptr(),
+                  nbytes, _stream(q))
   return out
 
 
@@ -219,19 +218,19 @@ def _linattn_block(x, w_qkv, b_qkv, w_out, b_out, head_num, kind, normalize_q):
     raise ValueError(f"weights need [{3 * C},{C}] and [{C},{C}] but got {tuple(w_qkv.shape)} and {tuple(w_out.shape)}")
   if (b_qkv is not None and tuple(b_qkv.shape) != (3 * C,)) or (b_out is not None and tuple(b_out.shape) != (C,)):
     raise ValueError(f"biases need [{3 * C}] and [{C}]")
-  lib = _lib.load()
-  x, w_qkv, w_out = x.contiguous(), w_qkv.contiguous(), w_out.contiguous()
-  b_qkv = None if b_qkv is None else b_qkv.contiguous()
-  b_out = None if b_out is None else b_out.contiguous()
+  ffi = _k()
+  for i, (name, t) in enumerate(tensors):
+    if t is not None and not t.is_contiguous():
+      raise ValueError(f"arg {i} ({name}) need a contiguous tensor but got strides {tuple(t.stride())}")
   y = torch.empty_like(x)
   dt = {torch.float16: _lib.FT_F16, torch.bfloat16: _lib.FT_BF16}.get(x.dtype, _lib.FT_F32)
-  a = _lib.FtLinBlockArgs(x.data_ptr(), w_qkv.data_ptr(), None if b_qkv is None else b_qkv.data_ptr(), w_out.data_ptr(),
-                          None if b_out is None else b_out.data_ptr(), y.data_ptr(), B, S, head_num, C // head_num, dt)
-  nbytes = lib.ft_linattn_block_workspace_bytes(ctypes.byref(a), kind)
+  a = ffi.LinBlockArgs(x.data_ptr(), w_qkv.data_ptr(), 0 if b_qkv is None else b_qkv.data_ptr(), w_out.data_ptr(),
+                       0 if b_out is None else b_out.data_ptr(), y.data_ptr(), B, S, head_num, C // head_num, dt)
+  nbytes = ffi.linattn_block_workspace_bytes(a, kind)
   if nbytes == 0:
-    _lib.check(_lib.FT_EUNSUPPORTED)
+    raise RuntimeError(f"libflashtensor_hip: {ffi.last_error()}")
   ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-  _lib.check(lib.ft_linattn_block_fwd(ctypes.byref(a), kind, int(bool(normalize_q)), ws.data_ptr(), nbytes, _stream(x)))
+  ffi.linattn_block_fwd(a, kind, int(bool(normalize_q)), ws.data_ptr(), nbytes, _stream(x))
   return y
 
 
@@ -250,23 +249,23 @@ def topk(score, k):
   """Indices [..., k] (int64) of the k largest entries along the last axis, descending."""
   if score.dtype != torch.float32 or not score.is_cuda:
     raise RuntimeError(f"arg 0 need a float32 GPU tensor but got {score.dtype} on {score.device}")
-  lib = _lib.load()
-  s = score.contiguous()
+  if not score.is_contiguous():
+    raise ValueError(f"arg 0 need a contiguous tensor but got strides {tuple(score.stride())}")
+  s = score
   S = s.shape[-1]
   rows = s.numel() // S
   idx = torch.empty(*s.shape[:-1], k, dtype=torch.int64, device=s.device)
-  _lib.check(lib.ft_topk(s.data_ptr(), rows, S, int(k), idx.data_ptr(), _stream(s)))
+  _k().topk(s.data_ptr(), rows, S, int(k), idx.data_ptr(), _stream(s))
   return idx
 
 
 def seeded_exp_rand(B, H, Sq, Skv, seed, device):
   """The noise tensor the seeded KeyFormer mode draws, materialised on `device` ("cpu" uses the host twin)."""
-  lib = _lib.load()
   device = torch.device(device)
   out = torch.empty(B, H, Sq, Skv, dtype=torch.float32, device=device)
   seed = int(seed) & 0xFFFFFFFFFFFFFFFF
   if device.type == "cpu":
-    _lib.check(lib.ft_noise_exp_fill_host(out.data_ptr(), B, H, Sq, Skv, seed))
+    _k().noise_exp_fill_host(out.data_ptr(), B, H, Sq, Skv, seed)
   else:
-    _lib.check(lib.ft_noise_exp_fill(out.data_ptr(), B, H, Sq, Skv, seed, _stream(out)))
+    _k().noise_exp_fill(out.data_ptr(), B, H, Sq, Skv, seed, _stream(out))
   return out

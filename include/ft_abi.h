@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FT_ABI_VERSION 4
+#define FT_ABI_VERSION 5
 
 enum FtStatus {
   FT_OK = 0,
@@ -117,7 +117,7 @@ int ft_avgpool1d(const float* src, int64_t rows, int32_t S, int32_t kernel, floa
 
 /* Linear attention cores of bench/ea.mlir:13-17 (kind = FT_OP_EA) and bench/sima.mlir:13-17 (FT_OP_SIMA):
  * O = f(Q) (g(K)^T V).  normalize_q applies SimA's L1 normalisation to Q as well (ignored for EA).
- * out_dtype: FtDtype of o (FT_F16/FT_BF16 = a->dtype, or FT_F32).  fp16 inputs; head_dim 64, or 32 (the
+ * out_dtype: FtDtype of o, FT_F16 or FT_F32.  fp16 inputs only (a->dtype == FT_F16); head_dim 64, or 32 (the
  * .mlir's own 4 heads of 32, :7-9) with an even number of heads stored 32 elements apart (s*.h == 32). */
 int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype, void* workspace,
                    size_t workspace_bytes, void* stream);
@@ -156,13 +156,6 @@ int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx
  * (ft_noise_exp_fill) or host memory (ft_noise_exp_fill_host). */
 int ft_noise_exp_fill(float* dst, int32_t B, int32_t H, int32_t Sq, int32_t Skv, uint64_t seed, void* stream);
 int ft_noise_exp_fill_host(float* dst, int32_t B, int32_t H, int32_t Sq, int32_t Skv, uint64_t seed);
-
-/* Diagnostic, no counterpart in the reference: what the matrix pipe sustains on given operand values.
- * `workgroups` workgroups of 8 waves each issue 4 * iters v_mfma_f32_32x32x16_f16 (32768 FLOP each) on fp16
- * fragments read from `operands` (64 KiB, any values) and nothing else; time the launch with events on the
- * stream.  clocks (optional, 2 x int64): shader-clock ticks and 100 MHz ticks one wave counted over its loop.
- * The chip is power-limited, so the rate depends on the bit patterns of the operands.  sink: >= 4 bytes, unused. */
-int ft_probe_mfma(const void* operands, int32_t workgroups, int32_t iters, float* sink, int64_t* clocks, void* stream);
 
 #ifdef __cplusplus
 }

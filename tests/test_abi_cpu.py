@@ -30,7 +30,9 @@ def test_library_exports_every_declared_symbol(lib):
   assert declared == sorted(_lib.EXPORTS)
   for name in declared:
     assert getattr(lib, name) is not None
-  assert lib.ft_abi_version() == 4 == _lib.ABI_VERSION
+  header = open(os.path.join(ROOT, "include", "ft_abi.h")).read()
+  version = int(re.search(r"#define FT_ABI_VERSION (\d+)", header).group(1))
+  assert lib.ft_abi_version() == version == _lib.ABI_VERSION
 
 
 def _args(**over):
@@ -158,11 +160,21 @@ def test_linear_block_argument_checks(lib):
   assert lib.ft_linattn_block_fwd(ctypes.byref(nul), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
 
 
-def test_probe_argument_checks(lib):
-  assert lib.ft_probe_mfma(None, 256, 10, 0x1000, None, None) == _lib.FT_EINVAL
-  assert lib.ft_probe_mfma(0x1008, 256, 10, 0x1000, None, None) == _lib.FT_EINVAL
-  assert lib.ft_probe_mfma(0x1000, 0, 10, 0x1000, None, None) == _lib.FT_EINVAL
-  assert lib.ft_probe_mfma(0x1000, 256, 0, 0x1000, None, None) == _lib.FT_EINVAL
+def test_diag_probe_is_outside_the_product_abi_and_checks_its_arguments(lib):
+  """The MFMA probe lives in libflashtensor_diag (include/ft_diag.h), not in the product library."""
+  assert not hasattr(lib, "ft_probe_mfma") and not hasattr(lib, "ft_diag_probe_mfma")
+  diag = _lib.load_diag()
+  big = 65536
+  assert diag.ft_diag_probe_mfma(None, big, 256, 10, 0x1000, None, None) == -1
+  assert b"null" in diag.ft_diag_last_error()
+  assert diag.ft_diag_probe_mfma(0x1008, big, 256, 10, 0x1000, None, None) == -1      # alignment
+  assert diag.ft_diag_probe_mfma(0x1000, big - 1, 256, 10, 0x1000, None, None) == -1  # operand buffer too small
+  assert b"FT_DIAG_PROBE_OPERAND_BYTES" in diag.ft_diag_last_error()
+  assert diag.ft_diag_probe_mfma(0x1000, big, 0, 10, 0x1000, None, None) == -1
+  assert diag.ft_diag_probe_mfma(0x1000, big, 256, 0, 0x1000, None, None) == -1
+  assert diag.ft_diag_probe_mfma(0x1000, big, 256, 4000001, 0x1000, None, None) == -1  # iteration cap
+  header = open(os.path.join(ROOT, "include", "ft_diag.h")).read()
+  assert "#define FT_DIAG_PROBE_OPERAND_BYTES 65536" in header and "#define FT_DIAG_PROBE_MAX_ITERS 4000000" in header
 
 
 def test_last_error_is_per_thread(lib):
@@ -220,8 +232,87 @@ def test_operator_layer_validates_like_the_reference_backend():
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
   monkeypatch.setattr(_lib, "_lib", None)
+  monkeypatch.setattr(_lib, "_ffi", None)
   monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libflashtensor_hip.so"))
   with pytest.raises(ImportError, match="not found"):
     _lib.load()
+  with pytest.raises(ImportError, match="not found"):
+    _lib.ffi()
   with pytest.raises(ImportError):
     ft.HipBuilder("attn").build_callable()
+
+
+# ------------------------------------------------------------------ the pybind11 module over the same ABI
+
+@pytest.fixture(scope="module")
+def ffi():
+  return _lib.ffi().kernels
+
+
+def test_ffi_module_binds_every_declared_entry_point(ffi):
+  """csrc/ffi_kernels.cpp exposes each function of include/ft_abi.h under its name without the ft_ prefix."""
+  for name in _declared():
+    assert callable(getattr(ffi, name[len("ft_"):])), name
+  assert ffi.abi_version() == ffi.ABI_VERSION == _lib.ABI_VERSION
+  assert (ffi.OK, ffi.EINVAL, ffi.EUNSUPPORTED, ffi.ELAUNCH, ffi.EWORKSPACE) == (0, -1, -2, -3, -4)
+  assert (ffi.F16, ffi.BF16, ffi.F32, ffi.CAUSAL, ffi.FAST_LOGITS) == (0, 1, 2, 1, 2)
+  assert (ffi.OP_ATTN, ffi.OP_COLSTATS, ffi.OP_KEYFORMER, ffi.OP_EA, ffi.OP_SIMA, ffi.OP_CORM) == (0, 1, 2, 3, 4, 5)
+
+
+def _ffi_args(ffi, **over):
+  st = (8 * 2 * 128, 2 * 128, 128)
+  base = dict(q=0x1000, k=0x2000, v=0x3000, o=0x4000, sq=st, sk=st, sv=st, so=st, B=1, H=2, Sq=8, Skv=8, D=128,
+              dtype=ffi.F16, flags=ffi.CAUSAL, Hkv=0)
+  base.update(over)
+  return ffi.AttnArgs(**base)
+
+
+@pytest.mark.parametrize("over,exc,needle", [
+    (dict(q=0), ValueError, "null"),
+    (dict(o=0), ValueError, "null"),
+    (dict(D=96), RuntimeError, "head_dim"),
+    (dict(dtype=2), RuntimeError, "dtype"),
+    (dict(Sq=0), ValueError, "shape"),
+    (dict(Sq=16, Skv=8), ValueError, "Skv >= Sq"),
+    (dict(q=0x1004), ValueError, "aligned"),
+    (dict(sq=(2048, 250, 128)), ValueError, "strides"),
+    (dict(H=6, Hkv=4), ValueError, "grouping"),
+])
+def test_ffi_module_maps_status_codes_to_exceptions(ffi, over, exc, needle):
+  """FT_EINVAL -> ValueError (std::invalid_argument), anything else -> RuntimeError (std::runtime_error), the
+  mapping of the reference's pybind layer (ffi/passes.cpp:81-83); nothing is launched for a rejected call."""
+  with pytest.raises(exc, match=needle) as info:
+    ffi.attn_fwd(_ffi_args(ffi, **over))
+  if exc is RuntimeError:
+    assert not isinstance(info.value, ValueError)
+  assert "status" in str(info.value)
+
+
+def test_ffi_module_workspace_and_validation_of_the_other_entry_points(ffi):
+  a = _ffi_args(ffi, B=2, H=4, Sq=100, Skv=100)
+  assert ffi.workspace_bytes(ffi.OP_ATTN, a) == 0
+  assert ffi.workspace_bytes(ffi.OP_COLSTATS, a) == 2 * 4 * 100 * 4
+  with pytest.raises(RuntimeError, match="workspace of 3200 bytes"):
+    ffi.attn_colstats_fwd(a, 0x5000, 0, 0x6000, 16)
+  with pytest.raises(ValueError, match="colsum"):
+    ffi.attn_colstats_fwd(a, 0, 0, 0x6000, 3200)
+  with pytest.raises(ValueError, match="tau"):
+    ffi.keyformer_fwd(a, ffi.Noise(seed=1), 0.0, 0x5000, 0x6000, 3200)
+  with pytest.raises(ValueError, match="softcap"):
+    ffi.attn_softcap_fwd(a, -1.0)
+  with pytest.raises(ValueError, match="odd"):
+    ffi.avgpool1d(0x1000, 4, 64, 4, 0x2000)
+  with pytest.raises(ValueError, match="top-k"):
+    ffi.topk(0x1000, 4, 64, 65, 0x2000)
+  with pytest.raises(RuntimeError, match="8192"):
+    ffi.topk(0x1000, 4, 8200, 8, 0x2000)
+  with pytest.raises(ValueError, match="kind"):
+    ffi.linattn_fwd(a, ffi.OP_ATTN, 1, ffi.F16, 0x6000, 1 << 20)
+  with pytest.raises(ValueError, match="3 entries"):
+    _ffi_args(ffi, sq=(1, 2))
+  # the host twin of the noise stream runs without a GPU and matches the oracle's integer arithmetic
+  import numpy as np
+  import oracle
+  buf = torch.empty(1, 2, 3, 5, dtype=torch.float32)
+  ffi.noise_exp_fill_host(buf.data_ptr(), 1, 2, 3, 5, 99)
+  np.testing.assert_allclose(buf.numpy(), oracle.seeded_exp_rand(99, 1, 2, 3, 5).numpy(), rtol=2e-6)

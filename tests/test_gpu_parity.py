@@ -332,9 +332,11 @@ def test_ea_sima_head_dim_32(gpu, B, S, H, seed):
   q2[:, :, 1], k2[:, :, 1], v2[:, :, 1] = q2[:, :, 1] * 3 + 1, k2[:, :, 1] * -2, v2[:, :, 1] + 5
   a, b = ops.ea(qd, kd, vd), ops.ea(q2, k2, v2)
   assert torch.equal(a[:, :, 0], b[:, :, 0]) and not torch.equal(a[:, :, 1], b[:, :, 1])
-  # a [B,H,S,D] storage order is made head-adjacent by the binding
+  # a [B,H,S,D] storage order does not have adjacent heads 32 elements apart: refused, not copied behind the caller's back
   qt = qd.transpose(1, 2).contiguous().transpose(1, 2)
-  assert torch.equal(ops.ea(qt, kd, vd), a)
+  if S > 1:
+    with pytest.raises(ValueError, match="32 elements apart"):
+      ops.ea(qt, kd, vd)
   with pytest.raises(RuntimeError, match="even number of heads"):
     ops.ea(qd[:, :, :1].contiguous(), kd[:, :, :1].contiguous(), vd[:, :, :1].contiguous())
 
@@ -622,7 +624,7 @@ def test_grouped_queries_2d(gpu, S, Skv, H, Hkv, D, masked):
   check_o(out, ref_o); check_score(score, ref_s)
   out_a = ft.kernels.Attn2D(Hkv, H, D, masked)(q.to(gpu), k.to(gpu), v.to(gpu))
   assert torch.equal(out_a, out)
-  assert torch.equal(out_a.cpu(), out_a.cpu()) and (out_a.float().cpu() - oracle.attn2d_forward(q, k, v, Hkv, H, D, masked).float()).abs().max() <= O_ABS
+  check_o(out_a, oracle.attn2d_forward(q, k, v, Hkv, H, D, masked))
 
 
 def test_grouped_queries_equal_repeated_kv_heads(gpu):
@@ -633,9 +635,9 @@ def test_grouped_queries_equal_repeated_kv_heads(gpu):
   assert torch.equal(out_g, out_r)                                         # same arithmetic, only the k/v addressing differs
   assert torch.allclose(s_g, s_r.view(2, 2, 4, 192).mean(dim=2), rtol=1e-6)
   assert torch.equal(ops.gemma2(qd, kg, vg), ops.gemma2(qd, kg.repeat_interleave(4, dim=2), vg.repeat_interleave(4, dim=2)))
-  with pytest.raises(ft._lib.FtError, match="grouped"):
+  with pytest.raises(RuntimeError, match="grouped"):
     ops.roco(qd, kg, vg)
-  with pytest.raises(ft._lib.FtError, match="grouped"):
+  with pytest.raises(RuntimeError, match="grouped"):
     ops.keyformer(qd, kg, vg, None, seed=1)
   with pytest.raises(RuntimeError, match="divisor"):
     ops.attn(qd, kd[:, :, :3].contiguous(), vd[:, :, :3].contiguous())
@@ -660,14 +662,48 @@ def test_config2_h2o_b1_h32_s2048_d128_with_topk(gpu):
   assert torch.allclose(s.sum(-1).cpu(), torch.full((1, 32), float(S)), rtol=1e-4)
 
 
-def test_config3_keyformer_b1_h32_s4096_d128_tau1(gpu):
-  S, H, HS = 4096, 32, 2  # oracle on the first HS heads
+# (b, h) pairs checked against the oracle at full size: first / last head of different XCD residues (workgroups
+# are dealt round-robin to the 8 XCDs, so head h of batch b lands on XCD (b H + h) % 8), first and last batch
+SPREAD_HEADS = (0, 7, 8, 15, 16, 23, 25, 31)
+
+
+def _take_pairs(t, pairs, head_axis):
+  """[1, len(pairs), ...] (head_axis 1) or [1, S, len(pairs), D] (head_axis 2) slices of chosen (b, h) pairs."""
+  if head_axis == 2:
+    return torch.stack([t[b, :, h] for b, h in pairs], dim=1).unsqueeze(0).contiguous()
+  return torch.stack([t[b, h] for b, h in pairs], dim=0).unsqueeze(0).contiguous()
+
+
+def test_headline_h2o_b1_h32_s4096_d128_with_topk(gpu):
+  """The benchmarked workload itself (H2O fp16, B1 H32 S4096 D128) against the oracle on 8 heads spread over
+  the XCDs, top-k k = S/8 by the gap rule, row-sum invariant on all heads."""
+  S, H = 4096, 32
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, 128, seed=0)
-  # seeded noise (the measured variant)
+  out, s = ops.h2o(qd, kd, vd)
+  idx = ops.topk(s, S // 8)
+  pairs = [(0, h) for h in SPREAD_HEADS]
+  sub = tuple(_take_pairs(t, pairs, 2) for t in (q, k, v))
+  ref_o, ref_s = oracle.chunked_over_heads(oracle.h2o_forward, sub, head_chunk=4)
+  check_o(_take_pairs(out.cpu(), pairs, 2), ref_o)
+  check_score(_take_pairs(s.cpu(), pairs, 1), ref_s)
+  assert oracle.topk_agreement(_take_pairs(idx.cpu(), pairs, 1), ref_s, S // 8) == 0
+  assert torch.allclose(s.sum(-1).cpu(), torch.full((1, H), float(S)), rtol=1e-4)
+  assert torch.equal(out[:, 0].cpu(), v[:, 0])
+
+
+def test_config3_keyformer_b1_h32_s4096_d128_tau1(gpu):
+  S, H = 4096, 32
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, 128, seed=0)
+  # seeded noise (the measured variant): oracle on 8 heads spread over the XCDs, 2 at a time (each head's
+  # eager KeyFormer holds several S x S fp32 tensors)
   out, s = ops.keyformer(qd, kd, vd, None, tau=1.0, seed=2024)
-  es = oracle.seeded_exp_rand(2024, 1, HS, S, S)
-  ref_o, ref_s = oracle.keyformer_forward(q[:, :, :HS].contiguous(), k[:, :, :HS].contiguous(), v[:, :, :HS].contiguous(), es, tau=1.0)
-  check_o(out[:, :, :HS], ref_o); check_score(s[:, :HS], ref_s)
+  pairs = [(0, h) for h in SPREAD_HEADS]
+  for i in range(0, len(pairs), 2):
+    pp = pairs[i:i + 2]
+    es = oracle.seeded_exp_rand_pairs(2024, H, pp, S, S)
+    ref_o, ref_s = oracle.keyformer_forward(*(_take_pairs(t, pp, 2) for t in (q, k, v)), es, tau=1.0)
+    check_o(_take_pairs(out.cpu(), pp, 2), ref_o); check_score(_take_pairs(s.cpu(), pp, 1), ref_s)
+    del es
   assert torch.allclose(s.sum(-1).cpu(), torch.full((1, H), float(S)), rtol=1e-4)
   # tensor noise: degenerate noise E == 1 at tau == 1 must reproduce the H2O score on all heads
   ones = torch.ones(1, H, S, S, dtype=torch.float32, device=gpu)
@@ -676,32 +712,49 @@ def test_config3_keyformer_b1_h32_s4096_d128_tau1(gpu):
   # (the two paths differ in how the row sums are accumulated: fp32 exps vs the fp16 P fed to the MFMA)
   assert torch.allclose(s_ones, s_h2o, rtol=2e-4, atol=1e-7)
   del ones
-  # tensor noise, reference recipe and default tau, oracle on the first heads
+  # tensor noise, reference recipe and default tau, oracle on the first and last heads
+  HS = 2
+  tp = [(0, 0), (0, 31)]
   er = oracle.prepare_exp_rand(1, HS, S, S, seed=1)
   big = torch.ones(1, H, S, S, dtype=torch.float32, device=gpu)
-  big[:, :HS] = er.to(gpu)
+  big[:, 0] = er[:, 0].to(gpu)
+  big[:, 31] = er[:, 1].to(gpu)
   _, s_t = ops.keyformer(qd, kd, vd, big, tau=1.5)
-  _, ref_t = oracle.keyformer_forward(q[:, :, :HS].contiguous(), k[:, :, :HS].contiguous(), v[:, :, :HS].contiguous(), er, tau=1.5)
-  check_score(s_t[:, :HS], ref_t)
+  _, ref_t = oracle.keyformer_forward(*(_take_pairs(t, tp, 2) for t in (q, k, v)), er, tau=1.5)
+  check_score(_take_pairs(s_t.cpu(), tp, 1), ref_t)
 
 
 def test_config4_roco_b4_h32_s4096_d128(gpu):
   B, S, H = 4, 4096, 32
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, 128, seed=0)
   out, s1, s2 = ops.roco(qd, kd, vd)
-  sl = (slice(3, 4), slice(None), slice(30, 32))  # last batch, last two heads
-  ref_o, r1, r2 = oracle.roco_forward(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous())
-  check_o(out[sl], ref_o); check_score(s1[3:4, 30:32], r1); check_score(s2[3:4, 30:32], r2)
+  # 8 (b, h) pairs: batches 0 and 3 plus one each of 1 and 2, heads on different XCD residues
+  pairs = [(0, 0), (0, 7), (0, 31), (1, 8), (2, 15), (3, 0), (3, 24), (3, 31)]
+  sub = tuple(_take_pairs(t, pairs, 2) for t in (q, k, v))
+  ref_o, r1, r2 = oracle.chunked_over_heads(oracle.roco_forward, sub, head_chunk=4)
+  check_o(_take_pairs(out.cpu(), pairs, 2), ref_o)
+  check_score(_take_pairs(s1.cpu(), pairs, 1), r1); check_score(_take_pairs(s2.cpu(), pairs, 1), r2)
   assert torch.allclose(s1.sum(-1).cpu(), torch.full((B, H), float(S)), rtol=1e-4)
   assert (s2 >= 0).all() and (s2 <= s1 * (1 + 1e-6)).all()
   assert torch.equal(out[:, 0].cpu(), v[:, 0])
+  # the mean / variance the configuration names, against the oracle's on the checked pairs
   mean, var = ft.kernels.RoCo.mean_var(s1, s2, S)
+  ref_mean, ref_var = oracle.roco_mean_var(r1, r2, S)
+  check_score(_take_pairs(mean.cpu(), pairs, 1), ref_mean)
+  got_var = _take_pairs(var.cpu(), pairs, 1)
+  # var = sumsq / S - mean^2 cancels where a key's probabilities are nearly constant over the rows: the bar is
+  # 1e-3 of the larger term (what the two inputs' own 1e-3 allow), i.e. relative to sumsq / S
+  assert ((got_var - ref_var).abs() <= 2e-3 * (r2 / S)).all()
   assert (var > -1e-7).all() and torch.allclose(mean.sum(-1).cpu(), torch.ones(B, H), rtol=1e-4)
-  # q == 0: uniform causal rows => harmonic-number closed forms at full size
+  # q == 0: uniform causal rows => harmonic-number closed forms at full size, mean / variance included
   _, z1, z2 = ops.roco(torch.zeros_like(qd[:1, :, :2]), kd[:1, :, :2], vd[:1, :, :2])
   inv = 1.0 / np.arange(1, S + 1)
-  assert np.abs(z1[0, 0].cpu().numpy() / np.cumsum(inv[::-1])[::-1] - 1).max() < 1e-4
-  assert np.abs(z2[0, 1].cpu().numpy() / np.cumsum((inv ** 2)[::-1])[::-1] - 1).max() < 1e-4
+  h1, h2 = np.cumsum(inv[::-1])[::-1], np.cumsum((inv ** 2)[::-1])[::-1]
+  assert np.abs(z1[0, 0].cpu().numpy() / h1 - 1).max() < 1e-4
+  assert np.abs(z2[0, 1].cpu().numpy() / h2 - 1).max() < 1e-4
+  zm, zv = ft.kernels.RoCo.mean_var(z1, z2, S)
+  assert np.abs(zm[0, 1].cpu().numpy() / (h1 / S) - 1).max() < 1e-4
+  assert np.abs(zv[0, 0].cpu().numpy() - (h2 / S - (h1 / S) ** 2)).max() < 1e-4 * (h2 / S).max()
 
 
 def test_config5_ea_sima_b8_h16_s8192_d64(gpu):
@@ -712,6 +765,61 @@ def test_config5_ea_sima_b8_h16_s8192_d64(gpu):
   o16 = ops.sima(qd, kd, vd)
   ref16 = oracle.sima_forward(q, k, v)
   assert (o16.float().cpu() - ref16.float()).abs().max().item() <= 1.2e-7  # two fp16 subnormal steps
+
+
+# ------------------------------------------------------------------ where the relaxed score bars come from
+
+def _kernel_logits(qd, kd, vd):
+  """The 16-bit logits f16(f16(QK^T) / sqrt(D)) exactly as the kernels round them, [B,H,Sq,Skv] fp16 on the host:
+  an unmasked problem with ONE key has p = 1, so its row normaliser is the logit itself (times log2 e), and an
+  MFMA result depends on its own row and column operands only, so the column-by-column values are the ones
+  every launch of the kernels sees for that (query, key) pair."""
+  cols = []
+  for j in range(kd.shape[1]):
+    _, lse = ops.attn(qd, kd[:, j:j + 1], vd[:, j:j + 1], causal=False, return_lse=True)
+    cols.append(lse)
+  t = torch.stack(cols, dim=-1).double() / float(np.log2(np.e))      # [B,H,Sq,Skv]
+  t16 = t.to(torch.float16)
+  assert (t16.double() - t).abs().max().item() < 1e-5                # an fp16 value to within fp32 rounding
+  return t16.cpu()
+
+
+@pytest.mark.parametrize("S,D,seed", [(520, 128, 61), (384, 64, 62)])
+def test_logit_rounding_flips_explain_the_relaxed_bars(gpu, S, D, seed):
+  """The CPU definition and the kernels accumulate QK^T in different orders; where a sum sits on an fp16
+  rounding boundary the 16-bit logit comes out one ulp apart.  Measured here instead of argued: (1) such
+  flips are rare and one ulp of QK^T each; (2) keys whose column holds no flip meet the plain 1e-3 bar; (3) with
+  the kernels' own logits fed to the CPU definition every key meets it, the last ones included."""
+  H = 2
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, D, seed=seed)
+  t_gpu = _kernel_logits(qd, kd, vd)                                  # [1,H,S,S] fp16
+  scores, probs = oracle.cases._masked_scores_probs(q, k)             # the CPU definition's masked fp16 logits
+  visible = torch.isfinite(scores)
+  assert visible.sum().item() == H * S * (S + 1) // 2
+  a, b = scores[visible].float(), t_gpu[visible].float()
+  flipped = a != b
+  n_flip = int(flipped.sum())
+  # One ulp of the fp16 QK^T, carried through the division by sqrt(D): a relative step in (2^-11, 2^-10], i.e.
+  # one or two ulps of the quotient (fp16 spacing 2^-10 * 2^floor(log2 |x|)).  Quotients below 2.5e-3 may also
+  # differ by 2e-6 (the packed form of the division by sqrt(128) is exact above that only).
+  ulp = torch.maximum(a.abs(), b.abs()).clamp_min(2.0 ** -14).log2().floor().exp2() * 2.0 ** -10
+  assert ((a - b).abs() <= 2.001 * ulp + 2e-6).all()
+  assert n_flip <= 4e-3 * a.numel(), f"{n_flip} of {a.numel()} logits differ"
+  _, s1, s2 = ops.roco(qd, kd, vd)
+  _, r1, r2 = oracle.roco_forward(q, k, v)
+  flip_map = torch.zeros_like(scores, dtype=torch.bool)
+  flip_map[visible] = flipped
+  clean = ~flip_map.any(dim=2)                                        # [1,H,S]: keys with no flipped logit in their column
+  assert clean.float().mean().item() > 0.2
+  e1 = ((s1.cpu() - r1).abs() / r1)[clean].max().item()
+  e2 = ((s2.cpu() - r2).abs() / r2)[clean].max().item()
+  assert e1 <= SCORE_REL and e2 <= 2 * SCORE_REL, (e1, e2)            # squares double a relative error
+  # the CPU definition evaluated on the kernels' logits (h2o.py:30-36 from `scores` on)
+  tg = t_gpu.clone()
+  tg[~visible] = float("-inf")
+  p_gpu = torch.softmax(tg.float(), dim=-1)
+  check_score(s1, p_gpu.sum(dim=2)); check_score(s2, (p_gpu * p_gpu).sum(dim=2), rel=2 * SCORE_REL)
+  print(f"S={S} D={D}: {n_flip} of {a.numel()} logits flipped; clean-key score error {e1:.2e} / {e2:.2e}")
 
 
 # ------------------------------------------------------------------ seeded random shapes
@@ -793,12 +901,13 @@ def test_calls_can_be_captured_in_a_hip_graph(gpu):
 def test_mfma_probe_runs_and_reports_clocks(gpu):
   import ctypes
   from flashtensor_amd import _lib
-  lib = _lib.load()
+  diag = _lib.load_diag()
   operands = torch.randn(32768, dtype=torch.float16, device=gpu)
   sink = torch.zeros(4, dtype=torch.float32, device=gpu)
   clocks = torch.zeros(2, dtype=torch.int64, device=gpu)
-  _lib.check(lib.ft_probe_mfma(operands.data_ptr(), 64, 2000, sink.data_ptr(), clocks.data_ptr(),
-                               ctypes.c_void_p(torch.cuda.current_stream(gpu).cuda_stream)))
+  rc = diag.ft_diag_probe_mfma(operands.data_ptr(), operands.numel() * 2, 64, 2000, sink.data_ptr(), clocks.data_ptr(),
+                               ctypes.c_void_p(torch.cuda.current_stream(gpu).cuda_stream))
+  assert rc == 0, diag.ft_diag_last_error()
   torch.cuda.synchronize()
   shader, wall = clocks.cpu().tolist()
   assert shader >= 2000 * 4 * 8 and wall > 0            # at least eight passes per MFMA... and the wall clock moved
@@ -819,3 +928,26 @@ def test_cli_builds_and_runs_every_case(gpu, capsys):
     first = res[0] if isinstance(res, tuple) else res
     assert torch.isfinite(first.float()).all(), name
     assert "hip" in capsys.readouterr().out
+
+
+def test_cli_check_prints_the_loss_lines_against_golden_outputs(gpu, capsys):
+  """`--check FILE.npz` prints the reference harness's loss(out, ref, remove_zero=True) lines
+  (cases/attn_h2o.py:144-145) against expected outputs from a golden file; the numbers must sit inside the bars."""
+  import ast
+  from flashtensor_amd import run as cli
+  plan = [("attn", "softmax_s128_d128.npz", [("abs_max", O_ABS)]),
+          ("h2o", "softmax_s200_d128.npz", [("abs_max", O_ABS), ("rel_max", SCORE_REL)]),
+          ("roco", "softmax_s256_d64.npz", [("abs_max", O_ABS), ("rel_max", SCORE_REL), ("rel_max", 2 * SCORE_REL)]),
+          ("snapkv", "next_s200_d64.npz", [("rel_max", SCORE_REL)]),
+          ("gemma2", "next_s128_d128.npz", [("abs_max", O_ABS)]),
+          ("ea", "linear_s200_d64.npz", [("abs_max", 2e-3)]),
+          ("sima", "linear_s256_d64.npz", [("rel_mean", 1e-3)])]
+  for name, fname, bars in plan:
+    cli.main(["-m", name, "--check", os.path.join(GOLDEN, fname), "--run", "1", "--warmup", "1"])
+    lines = [ln for ln in capsys.readouterr().out.splitlines() if ln.startswith("loss(out[")]
+    assert len(lines) == len(bars), (name, lines)
+    for ln, (key, bar) in zip(lines, bars):
+      got = ast.literal_eval(ln.split(")=", 1)[1])
+      assert got["remove_zero"] is True and got[key] <= bar, (name, ln)
+  with pytest.raises(SystemExit, match="--check knows"):
+    cli.main(["-m", "corm", "--check", os.path.join(GOLDEN, "next_s128_d128.npz")])
