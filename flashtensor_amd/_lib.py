@@ -18,7 +18,7 @@ FT_OP_ATTN, FT_OP_COLSTATS, FT_OP_KEYFORMER, FT_OP_EA, FT_OP_SIMA, FT_OP_CORM = 
 ABI_VERSION = 5
 
 # every symbol include/ft_abi.h declares
-EXPORTS = ("ft_abi_version", "ft_last_error", "ft_workspace_bytes", "ft_attn_fwd", "ft_attn_colstats_fwd",
+EXPORTS = ("ft_abi_version", "ft_last_error", "ft_workspace_bytes", "ft_attn_fwd", "ft_attn_colstats_fwd", "ft_attn_colstats_fwd_static",
            "ft_keyformer_fwd", "ft_attn_softcap_fwd", "ft_corm_fwd", "ft_avgpool1d", "ft_linattn_fwd", "ft_topk",
            "ft_noise_exp_fill", "ft_noise_exp_fill_host", "ft_linattn_block_workspace_bytes", "ft_linattn_block_fwd")
 
@@ -78,6 +78,8 @@ def load():
   lib.ft_attn_fwd.argtypes = [args_p, f32p, vp]
   lib.ft_attn_colstats_fwd.restype = ctypes.c_int
   lib.ft_attn_colstats_fwd.argtypes = [args_p, f32p, f32p, vp, ctypes.c_size_t, vp]
+  lib.ft_attn_colstats_fwd_static.restype = ctypes.c_int
+  lib.ft_attn_colstats_fwd_static.argtypes = [args_p, f32p, f32p, vp]
   lib.ft_keyformer_fwd.restype = ctypes.c_int
   lib.ft_keyformer_fwd.argtypes = [args_p, noise_p, ctypes.c_float, f32p, vp, ctypes.c_size_t, vp]
   lib.ft_attn_softcap_fwd.restype = ctypes.c_int

@@ -275,6 +275,30 @@ int run_colstats(const FtAttnArgs* a, float* colsum, float* colsumsq, void* ws, 
   return FT_OK;
 }
 
+// Scratch of ft_attn_colstats_fwd_static: device memory that is part of the loaded code object, so that the
+// entry point never calls an allocator.  Each GPU holds its own copy at its own address; the name below is a
+// host-side handle, not a device address: the address is looked up once per device (with that device current)
+// and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[FT_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];  // zero-initialised; a racing first call stores the same address twice
+
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(FT_EUNSUPPORTED, "device index %d beyond the %d this entry point tracks", dev, kMaxDevices);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return FT_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -319,6 +343,17 @@ int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, vo
     return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
   if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(FT_EINVAL, "workspace must be 4-byte aligned");
   return run_colstats(a, colsum, colsumsq, workspace, stream);
+}
+
+int ft_attn_colstats_fwd_static(const FtAttnArgs* a, float* colsum, float* colsumsq, void* stream) {
+  if (int rc = validate_colstats(a, colsum, colsumsq)) return rc;
+  const size_t need = colstats_bytes(a);
+  if (need > (size_t)FT_STATIC_SCRATCH_BYTES)
+    return fail(FT_EWORKSPACE, "problem needs %zu bytes of scratch, the static buffer holds %zu: use ft_attn_colstats_fwd with a workspace",
+                need, (size_t)FT_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return run_colstats(a, colsum, colsumsq, ws, stream);
 }
 
 int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float* kf_score, void* workspace,

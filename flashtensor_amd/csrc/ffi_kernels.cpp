@@ -59,6 +59,7 @@ void init_ffi_kernels(py::module_&& m) {
   m.attr("OP_EA") = (int)FT_OP_EA;
   m.attr("OP_SIMA") = (int)FT_OP_SIMA;
   m.attr("OP_CORM") = (int)FT_OP_CORM;
+  m.attr("STATIC_SCRATCH_BYTES") = (size_t)FT_STATIC_SCRATCH_BYTES;
 
   py::class_<FtAttnArgs>(m, "AttnArgs", py::module_local())
       .def(py::init([](uintptr_t q, uintptr_t k, uintptr_t v, uintptr_t o, py::tuple sq, py::tuple sk, py::tuple sv, py::tuple so,
@@ -106,6 +107,11 @@ void init_ffi_kernels(py::module_&& m) {
     py::gil_scoped_release nogil;
     check(ft_attn_colstats_fwd(&a, ptr<float>(colsum), ptr<float>(colsumsq), ptr<void>(ws), ws_bytes, ptr<void>(stream)));
   }, py::arg("args"), py::arg("colsum"), py::arg("colsumsq"), py::arg("workspace"), py::arg("workspace_bytes"), py::arg("stream") = 0);
+
+  m.def("attn_colstats_fwd_static", [](const FtAttnArgs& a, uintptr_t colsum, uintptr_t colsumsq, uintptr_t stream) {
+    py::gil_scoped_release nogil;
+    check(ft_attn_colstats_fwd_static(&a, ptr<float>(colsum), ptr<float>(colsumsq), ptr<void>(stream)));
+  }, py::arg("args"), py::arg("colsum"), py::arg("colsumsq") = 0, py::arg("stream") = 0);
 
   m.def("keyformer_fwd", [](const FtAttnArgs& a, const FtNoise& noise, float tau, uintptr_t kf_score, uintptr_t ws, size_t ws_bytes,
                             uintptr_t stream) {

@@ -91,6 +91,16 @@ int ft_attn_fwd(const FtAttnArgs* a, float* lse, void* stream);
 int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* ft_attn_colstats_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): no workspace argument; the row normalisers (and the per-head
+ * sums of grouped queries) live in a static device buffer of FT_STATIC_SCRATCH_BYTES that the library's code object
+ * carries on every GPU it is loaded on.  No counterpart in the reference.  Problems whose
+ * ft_workspace_bytes(FT_OP_COLSTATS, a) exceeds the buffer are refused with FT_EWORKSPACE.  Calls no allocator.
+ * All calls on one GPU share that GPU's buffer: two calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream are ordered.  Results are those of ft_attn_colstats_fwd, bit for bit. */
+#define FT_STATIC_SCRATCH_BYTES (8u << 20)
+int ft_attn_colstats_fwd_static(const FtAttnArgs* a, float* colsum, float* colsumsq, void* stream);
+
 /* KeyFormer.forward (cases/kernels/kf.py:19-42): attention + column sums of softmax((logits + gumbel)/tau),
  * gumbel = -log(exp_rand).  kf_score: [B,H,Skv] fp32. */
 int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float* kf_score, void* workspace,
