@@ -24,6 +24,7 @@
 namespace ft {
 
 constexpr int kAttnBN = 64;
+constexpr bool kAttnTwoBlocks = true;
 
 // Rescale threshold of the running maximum in log2 units: the stale maximum is kept (and O, l are not
 // rescaled) while the new row maximum exceeds it by less than this, so unnormalised probabilities stay
@@ -75,9 +76,16 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     mb = rank < half ? nMB - 1 - rank : rank - half;
   }
   const int b = bh / p.H, h = bh % p.H;
-  const int m0 = mb * BM;
   const int lane = lane_id(), wave = wave_id();
   const int g = lane >> 5, n = lane & 31;
+  // two_blocks (causal, set by the launcher when the pairs fill the chip evenly): the workgroup takes query
+  // block nMB - 1 - slot and then block slot, the heaviest with the lightest, so that every workgroup walks the
+  // same number of key tiles and no workgroup is launched into a half-empty chip at the end
+  const int npass = (p.two_blocks && 2 * (int)(blockIdx.x / BH) != nMB - 1) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+  if (p.two_blocks) mb = pass == 0 ? nMB - 1 - (int)(blockIdx.x / BH) : (int)(blockIdx.x / BH);
+  if (pass) __syncthreads();  // every wave has left the first block's K/V tiles
+  const int m0 = mb * BM;
   const int qi = m0 + wave * 32 + n;
   const int qi_c = qi < p.Sq ? qi : p.Sq - 1;
   const float NEG_INF = -__builtin_inff();
@@ -592,6 +600,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     const float base = KF == kKfSeededTau1 ? m_run : KF == kKfSeededFast ? m_run * p.inv_tau : m_kf;
     if (qi < p.Sq && g == 0) p.lse_kf[(int64_t)bh * p.Sq + qi] = base + __builtin_amdgcn_logf(l_kf);
   }
+  }  // pass
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -616,10 +625,18 @@ static hipError_t launch_one(const AttnKernelParams& p0, hipStream_t stream) {
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
   // there are half as many of them: used on the pipelined paths once they still fill the chip twice
   constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast;
+  p.two_blocks = 0;
   if constexpr (kHas8) {
-    const int64_t n8 = (int64_t)((p.Sq + 255) / 256) * p.B * p.H;
-    if (n8 >= 2 * (int64_t)device_cu_count()) {
-      hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 8>), dim3((unsigned)n8), dim3(512), 0, stream, p);
+    const int nMB8 = (p.Sq + 255) / 256;
+    const int64_t n8 = (int64_t)nMB8 * p.B * p.H;
+    const int64_t cus = device_cu_count();
+    if (n8 >= 2 * cus) {
+      // causal: pair the heaviest block with the lightest inside one workgroup when the pairs come out as whole
+      // rounds of the chip (or as many rounds that a ragged last one does not matter)
+      const int64_t pairs = (int64_t)((nMB8 + 1) / 2) * p.B * p.H;
+      p.two_blocks = kAttnTwoBlocks && CAUSAL && nMB8 >= 2 && (pairs % cus == 0 || pairs >= 8 * cus);
+      const int64_t grid = p.two_blocks ? pairs : n8;
+      hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 8>), dim3((unsigned)grid), dim3(512), 0, stream, p);
       return hipGetLastError();
     }
   }

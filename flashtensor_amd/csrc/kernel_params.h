@@ -31,6 +31,7 @@ struct AttnKernelParams {
   float softcap;    // kKfSoftcap: logits become softcap * tanh(logit / softcap)
   int pair_order;   // block order of the causal attention kernel: heavy half descending, light half ascending
   int group;        // query heads per k/v head: query head h reads k/v head h / group
+  int two_blocks;   // 256-row form: a workgroup takes query blocks nMB - 1 - slot and slot (set by the launcher)
 };
 
 struct ColstatsKernelParams {
