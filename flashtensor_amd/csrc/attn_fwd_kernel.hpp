@@ -83,9 +83,12 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // two_blocks (causal, set by the launcher when the pairs fill the chip evenly): the workgroup takes query
   // block nMB - 1 - slot and then block slot, the heaviest with the lightest, so that every workgroup walks the
   // same number of key tiles and no workgroup is launched into a half-empty chip at the end
-  const int npass = (p.two_blocks && 2 * (int)(blockIdx.x / BH) != nMB - 1) ? 2 : 1;
+  // (compiled in only where the second pass costs no registers: with it the 4-wave form and the packed KeyFormer
+  // modes spill, and a spilled register's reload waits for the tile loads in flight: both count in vmcnt)
+  constexpr bool kTwoPass = WAVES == 8 && (KF == kKfNone || KF == kKfSoftcap);
+  const int npass = (kTwoPass && p.two_blocks && 2 * (int)(blockIdx.x / BH) != nMB - 1) ? 2 : 1;
   for (int pass = 0; pass < npass; ++pass) {
-  if (p.two_blocks) mb = pass == 0 ? nMB - 1 - (int)(blockIdx.x / BH) : (int)(blockIdx.x / BH);
+  if (kTwoPass && p.two_blocks) mb = pass == 0 ? nMB - 1 - (int)(blockIdx.x / BH) : (int)(blockIdx.x / BH);
   if (pass) __syncthreads();  // every wave has left the first block's K/V tiles
   const int m0 = mb * BM;
   const int qi = m0 + wave * 32 + n;
@@ -552,11 +555,12 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // pairs (it, it+1) of mask-free tiles whose staged tiles K[it+2], K[it+3], V[it+1], V[it+2] are whole tiles
   const int nf2 = max(0, min(n_fast, p.Skv / BN - 2)) & ~1;
   if constexpr (kFastMasked) {
-    // tiles from nf2 on go through the masked instance (which is exact for a tile that needs no mask as well)
-    if (nf2 > 0)
-      pend_max = tile_max(std::false_type{}, S0, 0);
-    else
-      pend_max = tile_max(std::true_type{}, S0, 0);
+    // tiles from nf2 on go through the masked instance (which is exact for a tile that needs no mask as well).
+    // Tile 0 always does: its maximum directly follows the MFMAs that produce the scores, and the mask-free instance
+    // reads them with hand-written v_max3 instructions, for which the compiler does not insert the wait states a
+    // vector instruction needs after the matrix instruction whose result it reads (in the loop sixteen PV MFMAs
+    // lie between the two); the masked instance reads them through ordinary selects first.
+    pend_max = tile_max(std::true_type{}, S0, 0);
   }
   for (; it < nf2 - 2; it += 2) {
     wait_vmem();
@@ -646,7 +650,7 @@ hipError_t launch_one(const AttnKernelParams& p0, hipStream_t stream) {
       // causal: pair the heaviest block with the lightest inside one workgroup when the pairs come out as whole
       // rounds of the chip (or as many rounds that a ragged last one does not matter)
       const int64_t pairs = (int64_t)((nMB8 + 1) / 2) * p.B * p.H;
-      p.two_blocks = kAttnTwoBlocks && CAUSAL && nMB8 >= 2 && (pairs % cus == 0 || pairs >= 8 * cus);
+      p.two_blocks = kAttnTwoBlocks && (KF == kKfNone || KF == kKfSoftcap) && CAUSAL && nMB8 >= 2 && (pairs % cus == 0 || pairs >= 8 * cus);
       const int64_t grid = p.two_blocks ? pairs : n8;
       hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 8>), dim3((unsigned)grid), dim3(512), 0, stream, p);
       return hipGetLastError();

@@ -298,6 +298,13 @@ def test_noise_stream_has_no_lattice_structure():
   assert stats.chisquare(pairs).pvalue > 1e-4
   pairs = np.bincount((u[:-1].flatten() * 64).astype(int) * 64 + (u[1:].flatten() * 64).astype(int), minlength=4096)
   assert stats.chisquare(pairs).pvalue > 1e-4
+  # the least significant bits that reach the uniform (bits 9..12 of the folded product; without the fold
+  # x ^= x >> 16 they fail this: bit k of a product depends on bits 0..k of its factors only): balanced, and
+  # independent between neighbours along either axis
+  low = (x >> np.uint32(9)) & np.uint32(15)
+  assert stats.chisquare(np.bincount(low.flatten(), minlength=16)).pvalue > 1e-4
+  assert stats.chisquare(np.bincount((low[:, :-1] * 16 + low[:, 1:]).flatten(), minlength=256)).pvalue > 1e-4
+  assert stats.chisquare(np.bincount((low[:-1] * 16 + low[1:]).flatten(), minlength=256)).pvalue > 1e-4
 
 
 # ------------------------------------------------------------------ SnapKV, CoRM, Gemma2
