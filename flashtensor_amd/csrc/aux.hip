@@ -22,9 +22,86 @@ __device__ __forceinline__ uint32_t float_order_desc(float x) {
   return ~u;                                       // flipped: larger scores first
 }
 
-__device__ __forceinline__ uint64_t lane_xor_u64(uint64_t v, int mask) {
-  const uint32_t lo = __shfl_xor((uint32_t)v, mask), hi = __shfl_xor((uint32_t)(v >> 32), mask);
+// Value of lane l ^ M for a compile-time M < 64, without the LDS crossbar a generic shuffle goes through (the sort is
+// a chain of ~60 dependent exchanges per row, so their latency is its run time): quad permutes for 1 and 2, half-row
+// mirror + quad reversal for 4 ((l ^ 7) ^ 3), a rotation by half a row for 8, v_permlane16_swap / v_permlane32_swap
+// for 16 and 32.
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor_u32(uint32_t v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "one bit of the lane index");
+  const int x = (int)v;
+  if constexpr (M == 1) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+  if constexpr (M == 2) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+  if constexpr (M == 4) {
+    const int h = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false);                         // row_half_mirror
+    return (uint32_t)__builtin_amdgcn_update_dpp(h, h, 0x1B, 0xF, 0xF, false);                       // quad_perm [3,2,1,0]
+  }
+  if constexpr (M == 8) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x128, 0xF, 0xF, false);  // row_ror:8
+  if constexpr (M == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);  // {rows 0,0,2,2}, {rows 1,1,3,3}
+    return (threadIdx.x & 16) ? (uint32_t)r[0] : (uint32_t)r[1];
+  }
+  if constexpr (M == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);  // {lower half twice}, {upper half twice}
+    return (threadIdx.x & 32) ? (uint32_t)r[0] : (uint32_t)r[1];
+  }
+#endif
+  return v;
+}
+
+template <int M>
+__device__ __forceinline__ uint64_t lane_xor_u64(uint64_t v) {
+  const uint32_t lo = lane_xor_u32<M>((uint32_t)v), hi = lane_xor_u32<M>((uint32_t)(v >> 32));
   return ((uint64_t)hi << 32) | lo;
+}
+
+// one compare-exchange step of the bitonic network at distance STRIDE inside runs of SIZE keys
+template <int E, int NT, int SIZE, int STRIDE>
+__device__ __forceinline__ void bitonic_step(uint64_t (&key)[E], uint64_t* xch, int t) {
+  if constexpr (STRIDE < E) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      if ((e & STRIDE) == 0) {
+        const bool up = ((t * E + e) & SIZE) == 0;
+        const uint64_t a = key[e], b = key[e | STRIDE];
+        const bool swap = (a > b) == up;
+        key[e] = swap ? b : a;
+        key[e | STRIDE] = swap ? a : b;
+      }
+    }
+  } else {
+    constexpr int M = STRIDE / E;  // partner thread t ^ M holds the partner of every key of this thread
+    const bool lower = (t & M) == 0;
+    if constexpr (M >= 64) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) xch[e * NT + t] = key[e];
+      __syncthreads();
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const uint64_t a = key[e];
+      uint64_t b;
+      if constexpr (M >= 64)
+        b = xch[e * NT + (t ^ M)];
+      else
+        b = lane_xor_u64<M>(a);
+      const bool up = ((t * E + e) & SIZE) == 0;
+      const bool want_min = lower == up;
+      key[e] = ((a < b) == want_min) ? a : b;
+    }
+    if constexpr (M >= 64) __syncthreads();
+  }
+}
+template <int E, int NT, int SIZE, int STRIDE>
+__device__ __forceinline__ void bitonic_merge(uint64_t (&key)[E], uint64_t* xch, int t) {
+  bitonic_step<E, NT, SIZE, STRIDE>(key, xch, t);
+  if constexpr (STRIDE > 1) bitonic_merge<E, NT, SIZE, STRIDE / 2>(key, xch, t);
+}
+template <int E, int NT, int SIZE>
+__device__ __forceinline__ void bitonic_sort(uint64_t (&key)[E], uint64_t* xch, int t) {
+  bitonic_merge<E, NT, SIZE, SIZE / 2>(key, xch, t);
+  if constexpr (SIZE < E * NT) bitonic_sort<E, NT, SIZE * 2>(key, xch, t);
 }
 
 template <int E, int NT>
@@ -39,41 +116,7 @@ __global__ void __launch_bounds__(NT) topk_kernel(const float* __restrict__ scor
     const int i = t * E + e;
     key[e] = i < S ? (((uint64_t)float_order_desc(row[i]) << 32) | (uint32_t)i) : ~0ull;  // padding sorts last
   }
-#pragma unroll
-  for (int size = 2; size <= N; size <<= 1) {
-#pragma unroll
-    for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      if (stride < E) {
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          if ((e & stride) == 0) {
-            const bool up = ((t * E + e) & size) == 0;
-            const uint64_t a = key[e], b = key[e | stride];
-            const bool swap = (a > b) == up;
-            key[e] = swap ? b : a;
-            key[e | stride] = swap ? a : b;
-          }
-        }
-      } else {
-        const int m = stride / E;  // partner thread t ^ m holds the partner of every key of this thread
-        const bool lower = (t & m) == 0;
-        if (m >= 64) {
-#pragma unroll
-          for (int e = 0; e < E; ++e) xch[e * NT + t] = key[e];
-          __syncthreads();
-        }
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          const uint64_t a = key[e];
-          const uint64_t b = m >= 64 ? xch[e * NT + (t ^ m)] : lane_xor_u64(a, m);
-          const bool up = ((t * E + e) & size) == 0;
-          const bool want_min = lower == up;
-          key[e] = ((a < b) == want_min) ? a : b;
-        }
-        if (m >= 64) __syncthreads();
-      }
-    }
-  }
+  bitonic_sort<E, NT, 2>(key, xch, t);
   int64_t* out = idx + (int64_t)blockIdx.x * k;
 #pragma unroll
   for (int e = 0; e < E; ++e) {
