@@ -252,6 +252,17 @@ def main():
   step_us = event_time_us(step)
   attn_tflops = flops / attn_us / 1e6
   host_us = host_us_per_call(dev)
+  # the same step on inputs that rotate through 8 sets of q, k, v (805 MB, more than the 256 MB memory-side cache
+  # holds), so that no launch finds its operands cached by the previous one
+  sets = [tuple(torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3)) for _ in range(8)]
+  turn = [0]
+
+  def cold_step():
+    turn[0] = (turn[0] + 1) % len(sets)
+    return ops.h2o(*sets[turn[0]])
+
+  cold_us = event_time_us(cold_step)
+  del sets
 
   result = {
       "metric": "fused attn+score (H2O) algorithmic TFLOP/s at S=4096, 1 GPU",
@@ -278,7 +289,7 @@ def main():
                    "us_per_launch": round(attn_us, 1), "algorithmic_flop_per_launch": flops,
                    "timed_launches": KERNEL_TIMING_ITERS},
       "kernels_us": {"attn_fwd_kernel": round(attn_us, 1), "colstats_kernel": round(step_us - attn_us, 1),
-                     "step_events": round(step_us, 1)},
+                     "step_events": round(step_us, 1), "step_events_cold_inputs": round(cold_us, 1)},
   }
   try:
     result["mfma_probe"] = mfma_probe(dev)
