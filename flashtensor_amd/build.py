@@ -23,7 +23,10 @@ HEADERS = ["device_common.hpp", "kernel_params.h", "noise.h", "attn_fwd_kernel.h
            os.path.join("..", "..", "include", "ft_diag.h")]
 # packed fp32 VALU ops are disabled on purpose: some forms have produced wrong results on this hardware
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument"]
+         "-Wno-unused-command-line-argument",
+         # registers, scratch and spills of every kernel, written next to its object (see _resources): a spilled
+         # register in a loop that keeps direct-to-LDS loads in flight costs far more than its reload
+         "-Rpass-analysis=kernel-resource-usage"]
 
 
 def _hipcc():
@@ -39,6 +42,26 @@ def _stale(target, deps):
   return any(os.path.getmtime(d) > t for d in deps)
 
 
+def _resources(stderr):
+  """{mangled kernel name: {"vgprs", "agprs", "scratch_bytes", "vgpr_spill", "sgpr_spill", "occupancy", "lds_bytes"}}
+  from the compiler's kernel-resource-usage remarks."""
+  import re
+  keys = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes", "VGPRs Spill": "vgpr_spill",
+          "SGPRs Spill": "sgpr_spill", "Occupancy [waves/SIMD]": "occupancy", "LDS Size [bytes/block]": "lds_bytes"}
+  out, cur = {}, None
+  for m in re.finditer(r"remark:\s+([A-Za-z][^:\n]*):\s+(\S+) \[-Rpass-analysis=kernel-resource-usage\]", stderr):
+    name, val = m.group(1).strip(), m.group(2)
+    if name == "Function Name":
+      cur = out.setdefault(val, {})
+    elif cur is not None and name in keys:
+      cur[keys[name]] = int(val)
+  return out
+
+
+def resources_path(src):
+  return os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".resources.json")
+
+
 def _compile(src, force):
   obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
   deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS]
@@ -48,6 +71,9 @@ def _compile(src, force):
   res = subprocess.run(cmd, capture_output=True, text=True)
   if res.returncode != 0:
     raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")
+  import json
+  with open(resources_path(src), "w") as f:
+    json.dump(_resources(res.stderr), f, indent=1, sort_keys=True)
   return obj, res.stderr
 
 
