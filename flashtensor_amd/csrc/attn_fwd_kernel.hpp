@@ -113,8 +113,9 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     nw = min(ntiles, (wave_row0 + 31 + p.off) / BN + 1);
     n_fast = min(n_fast, (wave_row0 + p.off + 1) / BN);  // tiles with n0 + BN - 1 <= wave_row0 + off
   }
-  if (!kFastMasked) n_fast = 0;  // only the pipelined path has a mask-free instance
   n_fast = min(n_fast, nw);
+  const int n_free = n_fast;             // leading tiles of which this wave sees every key
+  if (!kFastMasked) n_fast = 0;          // the pipelined loop (and its mask-free instance) is not used
 
   NoiseKeys nk = {0, 0};
   uint32_t a_i = 0;
@@ -360,84 +361,91 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     for (int i = 0; i < 4; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
   };
 
-  // ---- softmax of one tile: s (raw accumulators) -> pb (16-bit unnormalised probabilities)
-  auto softmax = [&](auto masked_tag, float16v (&s)[2], vec8 (&pb)[4], int n0, int buf, const float (&er)[2][16]) {
+  // ---- generic path (tensor-noise KeyFormer, and the seeded modes outside the packed form): softmax of one
+  // 32-key half of a tile, s (raw accumulators of one 32x32 block) -> pb (two MFMA operands of 16-bit
+  // unnormalised probabilities).  Half a tile at a time keeps the live set small enough for the noise slice
+  // of the next tile to be in flight beside the accumulators.
+  // MASKED: some key of the half is hidden from some query of the wave (the diagonal, the end of K).
+  auto softmax_half = [&](auto masked_tag, const float16v& s, vec8 (&pb)[2], int n0h, int buf, int mbk, const float (&er)[16]) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    // ---- logits in the log2 domain, with the reference's rounding points when EMU
-    const int jmax = CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1;  // last key this query sees
-    float rowmax = NEG_INF;
+    // ---- logits in the log2 domain, with the reference's rounding points when EMU (the same chains as the
+    // pipelined path: two elements per conversion)
+    float x[16];
+    if constexpr (EMU && kIsF16) {
+      const half2v pk_hi = __builtin_bit_cast(half2v, p.pk_hi2), pk_lo = __builtin_bit_cast(half2v, p.pk_lo2);
 #pragma unroll
-    for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = s[mbk][r];
-        if (EMU) {
-          x = T::to_float(T::from_float(x));
-          x = T::to_float(T::from_float(x * p.logit_mul));
-          if (KF == kKfSoftcap) {  // three 16-bit tensor ops in the reference (cases/kernels/gemma2.py:31-33)
-            x = T::to_float(T::from_float(x / p.softcap));
-            x = T::to_float(T::from_float(tanh_f32(x)));
-            x = T::to_float(T::from_float(x * p.softcap));
-          }
-          x *= kLog2e;
-        } else if (KF == kKfSoftcap) {
-          x = p.softcap * tanh_f32(x * (p.logit_mul * (1.f / kLog2e)) / p.softcap) * kLog2e;
-        } else {
-          x *= p.logit_mul;
-        }
-        if (MASKED) {
-          const int j = n0 + 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
-          x = (j > jmax) ? NEG_INF : x;
-        }
-        s[mbk][r] = x;
-        rowmax = fmaxf(rowmax, x);
+      for (int i = 0; i < 8; ++i) {
+        const float2v a2 = {s[2 * i], s[2 * i + 1]};
+        const half2v h2 = __builtin_convertvector(a2, half2v);  // QK^T is an fp16 tensor in the reference
+        // ... divided by sqrt(D) in fp16: t2 = 8 * f16(h / sqrt(D)), exact for D = 64, two packed ops for D = 128
+        const half2v t2 = D == 64 ? h2 : __builtin_elementwise_fma(h2, pk_hi, h2 * pk_lo);
+        x[2 * i] = (float)t2[0] * (kLog2e / 8.f);
+        x[2 * i + 1] = (float)t2[1] * (kLog2e / 8.f);
       }
+    } else if constexpr (EMU) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t h2 = T::pack2(s[2 * i], s[2 * i + 1]);
+        const uint32_t t2 = T::pack2(T::lo(h2) * p.logit_mul, T::hi(h2) * p.logit_mul);
+        x[2 * i] = T::lo(t2) * kLog2e;
+        x[2 * i + 1] = T::hi(t2) * kLog2e;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) x[r] = s[r] * p.logit_mul;
+    }
+    if (MASKED) {
+      // local key index of register r is 8 (r / 4) + 4 g + r % 4; it is visible iff <= lim + 4 g
+      const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0h - 4 * g;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) x[r] = (8 * (r >> 2) + (r & 3) > lim) ? NEG_INF : x[r];
+    }
+    float rowmax = max3(x[0], x[1], x[2]);
+#pragma unroll
+    for (int r = 3; r < 15; r += 2) rowmax = max3(rowmax, x[r], x[r + 1]);
+    rowmax = fmaxf(rowmax, x[15]);
     rowmax = fmaxf(rowmax, xchg32(rowmax));
 
     // ---- KeyFormer: running normaliser of softmax((logit + gumbel) / tau), gumbel = -ln(E)
-    if (KF == kKfTensor || KF == kKfSeeded) {
-      float z[2][16];
-      float zmax = NEG_INF;
+    {
+      float z[16];
 #pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float log2E;
-          if (KF == kKfTensor) {
-            log2E = __builtin_amdgcn_logf(er[mbk][r]);
-          } else {
-            const int jl = 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
-            const float u = noise_uniform(a_i, ldsCol[buf * BN + jl]);
-            log2E = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(u));
-          }
-          const float zz = (s[mbk][r] - log2E) * p.inv_tau;
-          z[mbk][r] = zz;
-          zmax = fmaxf(zmax, zz);
+      for (int r = 0; r < 16; ++r) {
+        float log2E;
+        if (KF == kKfTensor) {
+          log2E = __builtin_amdgcn_logf(er[r]);
+        } else {
+          const int jl = 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
+          const float u = noise_uniform(a_i, ldsCol[buf * BN + jl]);
+          log2E = __builtin_amdgcn_logf(-kLn2 * __builtin_amdgcn_logf(u));
         }
+        z[r] = (x[r] - log2E) * p.inv_tau;
+      }
+      float zmax = max3(z[0], z[1], z[2]);
+#pragma unroll
+      for (int r = 3; r < 15; r += 2) zmax = max3(zmax, z[r], z[r + 1]);
+      zmax = fmaxf(zmax, z[15]);
       zmax = fmaxf(zmax, xchg32(zmax));
+      // finite from the first half on: key 0 is visible to every row, so a later half that is hidden
+      // entirely (zmax = -inf) adds exp2(-inf) = 0
       const float mk_new = fmaxf(m_kf, zmax);
       float zs = 0.f;
 #pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) zs += __builtin_amdgcn_exp2f(z[mbk][r] - mk_new);
+      for (int r = 0; r < 16; ++r) zs += __builtin_amdgcn_exp2f(z[r] - mk_new);
       l_kf = l_kf * __builtin_amdgcn_exp2f(m_kf - mk_new) + zs;
       m_kf = mk_new;
     }
 
     rescale(rowmax);
-    uint4v pw[4];
+    uint4v pw[2];
 #pragma unroll
-    for (int mbk = 0; mbk < 2; ++mbk)
+    for (int r = 0; r < 16; r += 2) {
+      const uint32_t w = T::pack2(__builtin_amdgcn_exp2f(x[r] - m_run), __builtin_amdgcn_exp2f(x[r + 1] - m_run));
+      l_run = T::add2(w, l_run);  // row sum of the 16-bit P the MFMA consumes
+      pw[r >> 3][(r & 7) >> 1] = w;
+    }
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const uint16_t b0 = T::from_float(__builtin_amdgcn_exp2f(s[mbk][r] - m_run));
-        const uint16_t b1 = T::from_float(__builtin_amdgcn_exp2f(s[mbk][r + 1] - m_run));
-        l_run += T::to_float(b0) + T::to_float(b1);
-        pw[2 * mbk + (r >> 3)][(r & 7) >> 1] = (uint32_t)b0 | ((uint32_t)b1 << 16);
-      }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
+    for (int i = 0; i < 2; ++i) pb[i] = __builtin_bit_cast(vec8, pw[i]);
   };
 
   // ---- O^T += V^T P^T (32 transposed LDS reads, 16 MFMAs)
@@ -514,33 +522,14 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 
   // One iteration = one barrier.  On entry K[it+1] and V[it] have been requested; K[it+2] and V[it+1] are
   // requested here, into the buffers every wave has finished reading.
-  float er[2][16];
-  auto sync_and_stage = [&](int it, bool active, char* k_dst, char* v_dst) {
+  auto sync_and_stage = [&](int it, char* k_dst, char* v_dst) {
     wait_vmem();
     __syncthreads();
-    // KeyFormer, tensor mode: fetch this lane's slice of the noise tile before the next tiles' staging
-    // loads are queued, so that waiting for it does not wait for them.
-    if (KF == kKfTensor && active) {
-      const int n0 = it * BN;
-#pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int j0 = n0 + 32 * mbk + 8 * q4 + 4 * g;
-          if (p.er_vec4 && j0 + 3 < p.Skv) {
-            float4v e4 = *reinterpret_cast<const float4v*>(er_row + j0);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) er[mbk][4 * q4 + e] = e4[e];
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) er[mbk][4 * q4 + e] = (j0 + e < p.Skv) ? er_row[j0 + e] : 1.f;
-          }
-        }
-    }
     stage_k(it + 2, k_dst);
     stage_v(it + 1, v_dst);
   };
 
+  if constexpr (kFastMasked) {
   // ---- prologue: K[0], V[0], K[1] in flight; scores of tile 0
   stage_k(0, ldsK0);
   stage_v(0, ldsV0);
@@ -554,14 +543,12 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // ---- mask-free tiles, two per trip so that the two score buffers swap roles without copies
   // pairs (it, it+1) of mask-free tiles whose staged tiles K[it+2], K[it+3], V[it+1], V[it+2] are whole tiles
   const int nf2 = max(0, min(n_fast, p.Skv / BN - 2)) & ~1;
-  if constexpr (kFastMasked) {
-    // tiles from nf2 on go through the masked instance (which is exact for a tile that needs no mask as well).
-    // Tile 0 always does: its maximum directly follows the MFMAs that produce the scores, and the mask-free instance
-    // reads them with hand-written v_max3 instructions, for which the compiler does not insert the wait states a
-    // vector instruction needs after the matrix instruction whose result it reads (in the loop sixteen PV MFMAs
-    // lie between the two); the masked instance reads them through ordinary selects first.
-    pend_max = tile_max(std::true_type{}, S0, 0);
-  }
+  // tiles from nf2 on go through the masked instance (which is exact for a tile that needs no mask as well).
+  // Tile 0 always does: its maximum directly follows the MFMAs that produce the scores, and the mask-free instance
+  // reads them with hand-written v_max3 instructions, for which the compiler does not insert the wait states a
+  // vector instruction needs after the matrix instruction whose result it reads (in the loop sixteen PV MFMAs
+  // lie between the two); the masked instance reads them through ordinary selects first.
+  pend_max = tile_max(std::true_type{}, S0, 0);
   for (; it < nf2 - 2; it += 2) {
     wait_vmem();
     __syncthreads();
@@ -579,25 +566,90 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     fast_tile(std::false_type{}, std::true_type{}, std::true_type{}, S1, S0, ldsK0, ldsV1, (it + 1) * BN, it + 1, ldsK1, ldsV0);
     it += 2;
   }
-  // ---- tiles that straddle the diagonal or the end of K (and every tile of the other variants)
+  // ---- tiles that straddle the diagonal or the end of K
   for (; it < nw; ++it) {
     const bool odd = it & 1;
-    sync_and_stage(it, true, odd ? ldsK1 : ldsK0, odd ? ldsV0 : ldsV1);
-    if constexpr (kFastMasked) {
-      fast_tile(std::true_type{}, std::true_type{}, std::false_type{}, S0, S1, odd ? ldsK0 : ldsK1, odd ? ldsV1 : ldsV0, it * BN, it, nullptr, nullptr);
+    sync_and_stage(it, odd ? ldsK1 : ldsK0, odd ? ldsV0 : ldsV1);
+    fast_tile(std::true_type{}, std::true_type{}, std::false_type{}, S0, S1, odd ? ldsK0 : ldsK1, odd ? ldsV1 : ldsV0, it * BN, it, nullptr, nullptr);
 #pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk) S0[mbk] = S1[mbk];
-    } else {
-      vec8 pb[4];
-      softmax(std::true_type{}, S0, pb, it * BN, it & 1, er);
-      pv(pb, odd ? ldsV1 : ldsV0);
-      sched_pv_alone();
-      qk(S0, odd ? ldsK0 : ldsK1);
-      sched_qk_alone();
-    }
+    for (int mbk = 0; mbk < 2; ++mbk) S0[mbk] = S1[mbk];
   }
   // ---- tiles entirely above this wave's diagonal: keep the workgroup's barriers and staging in step
-  for (; it < ntiles; ++it) sync_and_stage(it, false, (it & 1) ? ldsK1 : ldsK0, (it & 1) ? ldsV0 : ldsV1);
+  for (; it < ntiles; ++it) sync_and_stage(it, (it & 1) ? ldsK1 : ldsK0, (it & 1) ? ldsV0 : ldsV1);
+  } else {
+  // ---- generic path: not pipelined across tiles.  K and V of tile it are read while those of tile it + 1 are
+  // loaded; a tile is worked on as two halves of 32 keys (8 + 8 MFMAs each), every key masked by comparison.
+  // Two tiles per trip, so that every LDS buffer is named at compile time: with a buffer chosen at run time
+  // the compiler cannot tell the tile being read from the tile being loaded, and drains every load in flight
+  // before the first LDS read of the tile.
+  // KeyFormer, tensor mode: er[mbk] is this lane's slice of the noise tile (its query row, the 16 keys of its
+  // score registers in half mbk).  The S x S tensor is the one operand that comes from HBM every time, so the
+  // slice of the next tile is requested as soon as the softmax has consumed this tile's (same registers) and is
+  // in flight for the rest of the tile: a load consumed in the iteration that issues it leaves the memory
+  // system idle while the tile is worked on.  (Ordinary loads: the four 16-byte pieces a lane pair takes from
+  // one 128-byte line arrive in four instructions, and with the non-temporal hint each went to HBM.)
+  float er[2][16];
+  auto load_er_half = [&](float (&dst)[16], int it, int mbk) __attribute__((always_inline)) {
+    const int c0 = it * BN + 32 * mbk;
+    if (p.er_vec4 && c0 + 32 <= p.Skv) {  // the whole half lies inside the tensor: four 16-byte loads
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const float4v e4 = *reinterpret_cast<const float4v*>(er_row + c0 + 8 * q4 + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[4 * q4 + e] = e4[e];
+      }
+    } else {  // keys past the end read the last one instead (no branches); they are masked
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst[r] = er_row[min(c0 + 8 * (r >> 2) + 4 * g + (r & 3), p.Skv - 1)];
+    }
+  };
+  auto qk_half = [&](float16v& s, const char* tk, int mbk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t)
+      s = T::mfma(*reinterpret_cast<const vec8*>(tk + koff[t] + mbk * 32 * G::RB), qf[t], s);
+  };
+  auto pv_half = [&](const vec8 (&pb)[2], const char* tv, int mbk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ksl = 0; ksl < 2; ++ksl)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma(read_vt(tv, 2 * mbk + ksl, db), pb[ksl], o_acc[db]);
+  };
+  auto slow_tile = [&](int it, auto odd_tag) __attribute__((always_inline)) {
+    constexpr bool odd = decltype(odd_tag)::value;
+    wait_vmem();
+    __syncthreads();
+    stage_k(it + 1, odd ? ldsK0 : ldsK1);
+    stage_v(it + 1, odd ? ldsV0 : ldsV1);
+    if (it < nw) {  // not entirely above this wave's diagonal
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) {
+        float16v s;
+        vec8 pb[2];
+        qk_half(s, odd ? ldsK1 : ldsK0, mbk);
+        if (it < n_free)
+          softmax_half(std::false_type{}, s, pb, it * BN + 32 * mbk, odd ? 1 : 0, mbk, er[mbk]);
+        else
+          softmax_half(std::true_type{}, s, pb, it * BN + 32 * mbk, odd ? 1 : 0, mbk, er[mbk]);
+        if (KF == kKfTensor && it + 1 < nw) load_er_half(er[mbk], it + 1, mbk);
+        pv_half(pb, odd ? ldsV1 : ldsV0, mbk);
+      }
+    }
+  };
+  if (KF == kKfTensor) {
+    load_er_half(er[0], 0, 0);
+    load_er_half(er[1], 0, 1);
+  }
+  stage_k(0, ldsK0);
+  stage_v(0, ldsV0);
+  int it = 0;
+  for (; it + 1 < ntiles; it += 2) {
+    slow_tile(it, std::false_type{});
+    slow_tile(it + 1, std::true_type{});
+  }
+  if (it < ntiles) slow_tile(it, std::false_type{});
+  }
 
   // ---- epilogue
   l_run += xchg32(l_run);

@@ -106,6 +106,40 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   auto stage_q = [&](int t, char* dst) {
     if (t < ntiles) stQ.issue(i_begin + t * BQ, min(BQ, p.Sq - (i_begin + t * BQ)), dst);
   };
+  // Tensor modes: this lane's slice of the S x S noise / threshold tensor for one tile (its key column, the rows
+  // of its score registers; 32 lanes read 128 contiguous bytes of a row), fetched one tile ahead of its use:
+  // the tensor is the only operand that comes from HBM every time, and a load consumed in the iteration that
+  // issues it leaves the memory system idle while the tile is worked on.  Tiles the causal mask hides from the
+  // wave are not read, and the loads carry the non-temporal hint: the tensor is read once and should not evict Q.
+  constexpr bool kTensor = MODE == kStatKfTensor || MODE == kStatCormTensor;
+  float er[2][16], er_nx[2][16];
+  auto load_er = [&](float (&dst)[2][16], int t) {
+    const int i0 = i_begin + t * BQ;
+    // nothing to fetch past the last tile, or when no row of the tile sees a key of this wave
+    if (t >= ntiles || (CAUSAL && wave_key0 > i0 + BQ - 1 + p.off)) return;
+    const float* row0 = er_col + (int64_t)(i0 + 4 * g) * p.er_sr;
+    if (i0 + BQ <= p.Sq && !(CAUSAL && wave_key0 + 31 > i0 + p.off)) {  // every pair of the tile is visible
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          dst[mbk][r] = __builtin_nontemporal_load(row0 + (int64_t)(32 * mbk + 8 * (r >> 2) + (r & 3)) * p.er_sr);
+    } else {
+      // Straddles the diagonal or the end of Q.  No branches and nothing that waits for a load here: a pair that
+      // does not exist (hidden by the mask, or past the last row) takes the element of the nearest visible pair of
+      // its key instead.  Its probability is zero, so the noise does not matter, and a threshold it could reach
+      // (<= 0) is reached by that visible pair as well.
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          int i = i0 + 4 * g + 32 * mbk + 8 * (r >> 2) + (r & 3);
+          if (CAUSAL) i = max(i, kj_c - p.off);
+          i = min(i, p.Sq - 1);
+          dst[mbk][r] = __builtin_nontemporal_load(er_col + (int64_t)i * p.er_sr);
+        }
+    }
+  };
   // rows of tile t: negated normaliser (-inf past Sq, so that those rows contribute exp2(-inf) = 0) and noise
   // row term.  The normaliser is fetched one iteration before it is parked in LDS, so that no wave sits
   // out a global-memory round trip inside the loop.
@@ -132,7 +166,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[mbk][r] = 0.f;
     // operand ring: reads run kAhead k-steps ahead of the MFMAs that consume them
-    constexpr int kAhead = 3;
+    constexpr int kAhead = kTensor ? 1 : 3;  // tensor modes: the registers go to the prefetched tensor slice
     vec8 qa[kAhead + 1][2];
 #pragma unroll
     for (int t = 0; t < kAhead; ++t)
@@ -155,16 +189,6 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
     constexpr bool MASKED = decltype(masked_tag)::value;
     const int buf = t & 1;
     const int i0 = i_begin + t * BQ;
-    float er[2][16];
-    if (MODE == kStatKfTensor || MODE == kStatCormTensor) {
-#pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = i0 + 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
-          er[mbk][r] = (i < p.Sq) ? er_col[(int64_t)i * p.er_sr] : 1.f;
-        }
-    }
     const half2v pk_hi = __builtin_bit_cast(half2v, p.pk_hi2), pk_lo = __builtin_bit_cast(half2v, p.pk_lo2);
     // key kj is hidden from row i0 + il when kj > i0 + il + off, i.e. il < lim
     const int lim = kj - i0 - p.off - 4 * g;
@@ -266,6 +290,7 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
   float16v S0[2], S1[2];
   if (ntiles > 0) {
     // ---- prologue: Q[0], Q[1] in flight; rows of tile 0; scores of tile 0
+    if (kTensor) load_er(er, 0);
     stage_q(0, ldsQ0);
     stage_q(1, ldsQ1);
     store_rows(0, load_rows(0));
@@ -276,10 +301,20 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
 
     // One iteration = one barrier.  On entry Q[t+1] has been requested and S0 (or S1) holds the scores of
     // tile t; Q[t+2] is requested into the buffer whose tile was consumed one iteration ago.
+    auto take_next_er = [&]() {
+      // nothing of the tile may be scheduled below this point: the wait for the prefetched slice (which, loads
+      // completing in order, is also a wait for the Q tile queued behind it) belongs at the very end
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) er[mbk][r] = er_nx[mbk][r];
+    };
     int t = 0;
     for (; t < n_masked; ++t) {
       wait_vmem();
       __syncthreads();
+      if (kTensor) load_er(er_nx, t + 1);  // ahead of the staging loads: waiting for it does not wait for them
       stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
       store_rows(t + 1, lse_next);
       lse_next = load_rows(t + 2);
@@ -287,6 +322,22 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, EMU, 
       const bool skip = CAUSAL && (wave_key0 > i_begin + t * BQ + BQ - 1 + p.off);
       if (!skip) reduce_tile(std::true_type{}, S0, t);
       qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
+      if (kTensor) take_next_er();
+    }
+    // Tensor modes are bound by the HBM stream of the tensor: one tile per trip, the registers of the second
+    // score buffer hold the prefetched slice instead.
+    if (kTensor) {
+      for (; t < ntiles; ++t) {
+        wait_vmem();
+        __syncthreads();
+        load_er(er_nx, t + 1);
+        stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
+        store_rows(t + 1, lse_next);
+        lse_next = load_rows(t + 2);
+        reduce_tile(std::false_type{}, S0, t);
+        qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
+        take_next_er();
+      }
     }
     // mask-free tiles, two per trip so that the score buffers swap roles without copies
     if ((ntiles - t) & 1) {  // make the remainder even with one single step
