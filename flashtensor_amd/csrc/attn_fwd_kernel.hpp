@@ -130,10 +130,10 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   TileStager<D, BN, NT, kTrSwizzle> stV;
   stK.init(kbase, p.sk.s);
   stV.init(vbase, p.sv.s);
-  auto stage_k = [&](int t, char* dst) {
+  auto stage_k = [&](int t, char* dst) __attribute__((always_inline)) {
     if (t < ntiles) stK.issue(t * BN, min(BN, p.Skv - t * BN), dst);
   };
-  auto stage_v = [&](int t, char* dst) {
+  auto stage_v = [&](int t, char* dst) __attribute__((always_inline)) {
     if (t < ntiles) stV.issue(t * BN, min(BN, p.Skv - t * BN), dst);
     if (kSeeded && t < ntiles && threadIdx.x < BN)
       ldsCol[(t & 1) * BN + threadIdx.x] = noise_col(nk, (uint32_t)(t * BN + threadIdx.x));
@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 
   // ---- S^T = K Q^T : [64 keys] x [32 queries] as two 32x32 blocks (16 LDS reads, 16 MFMAs), optionally
   // in two halves over the head dimension so that other work can sit between them
-  auto qk_part = [&](float16v (&s)[2], const char* tk, auto t0_tag, auto t1_tag) {
+  auto qk_part = [&](float16v (&s)[2], const char* tk, auto t0_tag, auto t1_tag) __attribute__((always_inline)) {
     constexpr int T0 = decltype(t0_tag)::value, T1 = decltype(t1_tag)::value;
     if (T0 == 0) {
 #pragma unroll
@@ -184,13 +184,13 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk) s[mbk] = T::mfma(ka[t][mbk], qf[t], s[mbk]);
   };
-  auto qk = [&](float16v (&s)[2], const char* tk) {
+  auto qk = [&](float16v (&s)[2], const char* tk) __attribute__((always_inline)) {
     qk_part(s, tk, std::integral_constant<int, 0>{}, std::integral_constant<int, KSTEPS>{});
   };
   // LDS latency is far longer than an MFMA, so operand reads must run several MFMAs ahead of their
   // consumers; sched_group_barrier sequences pin that order (the scheduler would otherwise sink each
   // read next to its use to save registers).  Masks: 0x008 MFMA, 0x100 LDS read, 0x002 VALU.
-  auto sched_qk_alone = [&]() {
+  auto sched_qk_alone = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
 #pragma unroll
     for (int t = 0; t < KSTEPS - 3; ++t) {
@@ -200,7 +200,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
   };
 
-  auto rescale = [&](float rowmax) {
+  auto rescale = [&](float rowmax) __attribute__((always_inline)) {
     const bool grow = rowmax > m_run + kRescaleSlack;  // identical in both lanes of a row
     if (__any(grow)) {
       const float m_new = grow ? rowmax : m_run;
@@ -224,10 +224,10 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // of a causal problem then has the normaliser of the reference, bit for bit).
   const float rcp_cap = kCap ? 1.f / p.softcap : 0.f;
   // row maximum of one tile's logits in the log2 domain (what rescale() compares with the running maximum)
-  auto tile_max = [&](auto masked_tag, const float16v (&s)[2], int n0) -> float {
+  auto tile_max = [&](auto masked_tag, const float16v (&s)[2], int n0) __attribute__((always_inline)) -> float {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const int lim = (CAUSAL ? min(qi + p.off, p.Skv - 1) : p.Skv - 1) - n0 - 4 * g;
-    auto at = [&](int mbk, int r) -> float {
+    auto at = [&](int mbk, int r) __attribute__((always_inline)) -> float {
       if (!MASKED) return s[mbk][r];
       const int jl = 32 * mbk + 8 * (r >> 2) + (r & 3);
       return jl > lim ? NEG_INF : s[mbk][r];
@@ -259,7 +259,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     return amax * p.logit_mul;  // logit_mul = log2e / sqrt(D) when the logits stay in fp32
   };
   // MASKED: key j of the tile is hidden from this lane's query when j > qi + off or j >= Skv.
-  auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0, int buf) {
+  auto fast_exp = [&](auto masked_tag, const float16v (&s)[2], vec8 (&pb)[4], int n0, int buf) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const float neg_m = -m_run;
     const half2v pk_hi = __builtin_bit_cast(half2v, p.pk_hi2), pk_lo = __builtin_bit_cast(half2v, p.pk_lo2);
@@ -449,14 +449,14 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   };
 
   // ---- O^T += V^T P^T (32 transposed LDS reads, 16 MFMAs)
-  auto read_vt = [&](const char* tv, int ks, int db) -> vec8 {
+  auto read_vt = [&](const char* tv, int ks, int db) __attribute__((always_inline)) -> vec8 {
     const char* p0 = tv + voff[db] + ks * 16 * G::RB;
     short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(FT_LDS(short4v, p0));
     short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(FT_LDS(short4v, p0 + 8 * G::RB));
     short8v both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(vec8, both);
   };
-  auto pv = [&](const vec8 (&pb)[4], const char* tv) {
+  auto pv = [&](const vec8 (&pb)[4], const char* tv) __attribute__((always_inline)) {
     vec8 va[4][DB];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
@@ -467,7 +467,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 #pragma unroll
       for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma(va[ks][db], pb[ks], o_acc[db]);
   };
-  auto sched_pv_alone = [&]() {
+  auto sched_pv_alone = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
 #pragma unroll
     for (int i = 0; i < 4 * DB - 4; ++i) {
@@ -485,7 +485,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   //   pend_max: log2-domain row maximum of the tile about to be processed (from the previous tile, or the prologue)
   float pend_max = NEG_INF;
   auto fast_tile = [&](auto masked_tag, auto next_masked_tag, auto stage_tag, float16v (&s_cur)[2], float16v (&s_next)[2],
-                       const char* tk_next, const char* tv, int n0, int it, char* k_dst, char* v_dst) {
+                       const char* tk_next, const char* tv, int n0, int it, char* k_dst, char* v_dst) __attribute__((always_inline)) {
     constexpr bool STAGE = decltype(stage_tag)::value;
     constexpr int kValuGroup = kKfFast ? 12 : kCap ? 11 : 6;  // vector instructions placed after each MFMA
     vec8 pb[4];
@@ -522,7 +522,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 
   // One iteration = one barrier.  On entry K[it+1] and V[it] have been requested; K[it+2] and V[it+1] are
   // requested here, into the buffers every wave has finished reading.
-  auto sync_and_stage = [&](int it, char* k_dst, char* v_dst) {
+  auto sync_and_stage = [&](int it, char* k_dst, char* v_dst) __attribute__((always_inline)) {
     wait_vmem();
     __syncthreads();
     stage_k(it + 2, k_dst);
@@ -567,6 +567,27 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     it += 2;
   }
   // ---- tiles that straddle the diagonal or the end of K
+  // Two per trip where the registers allow it (`it` is even here), so that the LDS buffers are named at compile
+  // time: with a buffer chosen at run time the compiler cannot tell the tile being read from the tile being
+  // loaded, and the first operand read of the tile waits for the K / V tiles requested a few instructions earlier.
+  constexpr bool kTailPairs = KF == kKfNone || KF == kKfSoftcap;
+  if constexpr (kTailPairs) {
+    auto tail_tile = [&](int it, auto odd_tag) __attribute__((always_inline)) {
+      constexpr bool odd = decltype(odd_tag)::value;
+      sync_and_stage(it, odd ? ldsK1 : ldsK0, odd ? ldsV0 : ldsV1);
+      fast_tile(std::true_type{}, std::true_type{}, std::false_type{}, S0, S1, odd ? ldsK0 : ldsK1, odd ? ldsV1 : ldsV0, it * BN, it, nullptr, nullptr);
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) S0[mbk] = S1[mbk];
+    };
+    for (; it + 1 < nw; it += 2) {
+      tail_tile(it, std::false_type{});
+      tail_tile(it + 1, std::true_type{});
+    }
+    if (it < nw) {
+      tail_tile(it, std::false_type{});
+      ++it;
+    }
+  }
   for (; it < nw; ++it) {
     const bool odd = it & 1;
     sync_and_stage(it, odd ? ldsK1 : ldsK0, odd ? ldsV0 : ldsV1);
