@@ -65,7 +65,9 @@ typedef struct FtAttnArgs {
 } FtAttnArgs;
 
 /* KeyFormer noise source.  exp_rand != NULL: the reference's input tensor [B,H,Sq,Skv] fp32
- * (cases/kernels/kf.py:19,36-37) with the given element strides (last axis contiguous).
+ * (cases/kernels/kf.py:19,36-37) with the given element strides (last axis contiguous); every element
+ * positive and finite, pairs hidden by the causal mask included: the reference adds -log(exp_rand) to the whole
+ * score matrix (kf.py:36-38), and the kernels may read any element of the tensor for a pair they then mask.
  * exp_rand == NULL: drawn in-kernel from the counter-based stream keyed by `seed`
  * (ft_noise_exp_fill* materialise the same tensor). */
 typedef struct FtNoise {
