@@ -140,6 +140,10 @@ struct StripMover {
       lds_off[it] = r * G::RB + c * 16;
     }
   }
+  // rows past `last` are read as row `last`: a wave that limits itself to its own share can issue every
+  // prefetch unconditionally (a fixed number of loads in flight, which the compiler can count: with loads that
+  // may or may not have been issued it waits for all of them) without touching another wave's rows
+  __device__ __forceinline__ void limit_rows(int last) { last_row = max(0, min(last_row, last)); }
   __device__ __forceinline__ void load(int row0, uint4v (&regs)[ROUNDS]) const {
 #pragma unroll
     for (int it = 0; it < ROUNDS; ++it) {
@@ -158,7 +162,7 @@ struct StripMover {
 template <bool EA, bool NQ>
 __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinParams p) {
   constexpr int D = kLinD, STEP = 16;
-  constexpr int P = 3;                        // strips in flight per wave
+  constexpr int P = NQ ? 2 : 3;               // strips in flight per wave (three tensors at three strips each do not fit in registers)
   constexpr int STRIP = STEP * 2 * D;         // 2 KB
   constexpr int R = STEP / 8;                 // 16-byte loads per lane, strip and tensor
   __shared__ __align__(16) char s_kv[kLinWaves][2 * STRIP];  // wave-private K and V strips
@@ -202,6 +206,12 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 
   uint4v rk[P][R], rv[P][R], rq[P][R];  // strips in flight, indexed by compile-time slot
   auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * STEP; };
+  {
+    const int last_mine = nmine > 0 ? strip_row0(nmine - 1) + STEP - 1 : tok_begin;
+    mvK.limit_rows(last_mine);
+    mvV.limit_rows(last_mine);
+    if (NQ) mvQ.limit_rows(last_mine);
+  }
   auto fetch = [&](int i, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     const int row0 = strip_row0(i);
@@ -305,9 +315,8 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
       for (int eb = 0; eb < 2; ++eb) acc[db][eb] = F16::mfma(ka[db], vb[eb], acc[db][eb]);
   };
 
-  // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P
-  // if this wave has one (a strip past its share would be another workgroup's rows: wasted HBM reads), then
-  // consume the parked strip
+  // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P (past
+  // the wave's share that re-reads its last row: see StripMover::limit_rows), then consume the parked strip
   auto step = [&](int i, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     const int t0 = strip_row0(i);
@@ -325,25 +334,35 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
         for (int e = 0; e < 8; ++e) qabs[e] += live ? __builtin_fabsf((float)qv[e]) : 0.f;
       }
     }
-    if (i + P < nmine) fetch(i + P, slot_tag);
+    fetch(i + P, slot_tag);
     wave_lds_order();
-    if (tail)
-      compute(std::true_type{}, t0);
-    else
-      compute(std::false_type{}, t0);
+    if (i < nmine) {
+      if (tail)
+        compute(std::true_type{}, t0);
+      else
+        compute(std::false_type{}, t0);
+    }
   };
 
-  if (0 < nmine) fetch(0, std::integral_constant<int, 0>{});
-  if (1 < nmine) fetch(1, std::integral_constant<int, 1>{});
-  if (2 < nmine) fetch(2, std::integral_constant<int, 2>{});
-  static_assert(P == 3, "the strip loop is unrolled over three register slots");
-  for (int i = 0; i < nmine;) {
+  // in this order (the scheduler is free to issue independent loads last-first, and loads complete in order: the
+  // first step would then wait for all three strips, and so would, after the compiler merges the two ways into
+  // the loop, every later one)
+  fetch(0, std::integral_constant<int, 0>{});
+  __builtin_amdgcn_sched_barrier(0);
+  fetch(1, std::integral_constant<int, 1>{});
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (P == 3) {
+    fetch(2, std::integral_constant<int, 2>{});
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // Whole trips of P steps (a step past the wave's share moves its re-read row and computes nothing): one
+  // entry, one back edge and the same loads on every path, so that the compiler knows how many are in flight at
+  // each step and waits for the oldest strip only.
+  static_assert(P == 2 || P == 3, "the strip loop is unrolled over the register slots");
+  for (int i = 0; i < nmine; i += P) {
     step(i, std::integral_constant<int, 0>{});
-    if (++i >= nmine) break;
-    step(i, std::integral_constant<int, 1>{});
-    if (++i >= nmine) break;
-    step(i, std::integral_constant<int, 2>{});
-    ++i;
+    step(i + 1, std::integral_constant<int, 1>{});
+    if constexpr (P == 3) step(i + 2, std::integral_constant<int, 2>{});
   }
 
   // ---- combine the four waves
@@ -610,13 +629,6 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   const int nsub = (tok_end - tok_begin + SUB - 1) / SUB;
   const int nmine = nsub > wave ? (nsub - wave + kLinWaves - 1) / kLinWaves : 0;
 
-  StripMover<SUB, kRowSwizzle> mvQ;
-  mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
-  uint4v rq[P][R];  // strips in flight, indexed by compile-time slot
-  auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * SUB; };
-  if (0 < nmine) mvQ.load(strip_row0(0), rq[0]);
-  if (1 < nmine) mvQ.load(strip_row0(1), rq[1]);
-
   // A operand: W^T[e][d], hi and lo, rows e = 32 eb + n, contraction slots d = 16 t + 8 g + [0..7]
   const uint16_t* w = p.w + (int64_t)bh * 2 * D * D;
   half8 whi[2][4], wlo[2][4];
@@ -627,6 +639,21 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
       whi[eb][t] = *reinterpret_cast<const half8*>(w + (32 * eb + n) * D + 16 * t + 8 * g);
       if (F32OUT) wlo[eb][t] = *reinterpret_cast<const half8*>(w + D * D + (32 * eb + n) * D + 16 * t + 8 * g);
     }
+
+  StripMover<SUB, kRowSwizzle> mvQ;
+  mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
+  uint4v rq[P][R];  // strips in flight, indexed by compile-time slot
+  auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * SUB; };
+  mvQ.limit_rows(nmine > 0 ? strip_row0(nmine - 1) + SUB - 1 : tok_begin);
+  __builtin_amdgcn_sched_barrier(0);  // W, then strip 0, then strip 1: loads complete in the order they are issued
+  mvQ.load(strip_row0(0), rq[0]);
+  __builtin_amdgcn_sched_barrier(0);
+  mvQ.load(strip_row0(1), rq[1]);
+  // W has landed before the loop starts, the two strips (the 2 R loads issued after it) stay in flight.  Left to
+  // the compiler, the wait for W sits inside the loop, in front of the MFMAs, where on every later trip it
+  // waits for the strip requested a few instructions earlier instead.
+  static_assert(P * R == 8, "the wait below counts the loads of the two strips");
+  __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8), every other counter at its maximum
   float winv[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) winv[i] = p.winv[bh * 4 + i];
@@ -634,16 +661,16 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   char* obase = static_cast<char*>(p.o) + (b * p.so.b + h * p.so.h) * (int64_t)(F32OUT ? 4 : 2);
   const int64_t orow_bytes = p.so.s * (int64_t)(F32OUT ? 4 : 2);
 
-  // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P
-  // if this wave has one (a strip past its share would be another workgroup's rows: wasted HBM reads), then
-  // consume the parked strip
+  // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P (past
+  // the wave's share that re-reads its last row: see StripMover::limit_rows), then consume the parked strip
   auto step = [&](int i, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     const int t0 = strip_row0(i);
     wave_lds_order();
     mvQ.to_lds(rq[SLOT], tq);
-    if (i + P < nmine) mvQ.load(strip_row0(i + P), rq[SLOT]);
+    mvQ.load(strip_row0(i + P), rq[SLOT]);
     wave_lds_order();
+    if (i >= nmine) return;  // past the wave's share: the slot has been moved and refilled, nothing to compute
 
     // B operand: f(Q)^T, column = token n, same contraction slots
     half8 qf[4];
@@ -750,11 +777,9 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   };
 
   static_assert(P == 2, "the strip loop is unrolled over two register slots");
-  for (int i = 0; i < nmine;) {
+  for (int i = 0; i < nmine; i += 2) {  // whole trips, as in the K/V pass
     step(i, std::integral_constant<int, 0>{});
-    if (++i >= nmine) break;
-    step(i, std::integral_constant<int, 1>{});
-    ++i;
+    step(i + 1, std::integral_constant<int, 1>{});
   }
 }
 
