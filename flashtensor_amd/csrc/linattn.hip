@@ -329,7 +329,7 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 #pragma unroll
       for (int it = 0; it < R; ++it) {
         const half8 qv = __builtin_bit_cast(half8, rq[SLOT][it]);
-        const bool live = !tail || t0 + it * 8 + (lane >> 3) < p.S;
+        const bool live = i < nmine && (!tail || t0 + it * 8 + (lane >> 3) < p.S);  // not a re-read row past the share
 #pragma unroll
         for (int e = 0; e < 8; ++e) qabs[e] += live ? __builtin_fabsf((float)qv[e]) : 0.f;
       }
