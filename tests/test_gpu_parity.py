@@ -476,6 +476,10 @@ def test_corm_small(gpu, B, S, H, D, seed):
   # all-ones thresholds keep only key 0
   k1 = ops.corm(qd, kd, vd, torch.ones(S, S, device=gpu))[1]
   assert k1[..., 0].all() and not k1[..., 1:].any()
+  # thresholds of pairs the causal mask hides take no part (in the reference p = 0 >= NaN is false as well)
+  holes = thr.clone()
+  holes[torch.triu(torch.ones(S, S, dtype=torch.bool), diagonal=1)] = float("nan")
+  assert torch.equal(ops.corm(qd, kd, vd, holes.to(gpu))[1], ops.corm(qd, kd, vd, thr.contiguous().to(gpu))[1])
 
 
 def test_corm_zero_queries_keep_every_key(gpu):
