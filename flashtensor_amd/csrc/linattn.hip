@@ -58,6 +58,7 @@ struct LinParams {
   int out_nch;              // the same for the output pass (its chunks are independent of the K/V pass's)
   int out_tiles_per_chunk;
   int half_heads;           // every 64-channel "head" is two adjacent heads of 32 channels (head_dim 32)
+  int out_wave_heads;       // output pass: a workgroup takes four adjacent heads, one per wave
 };
 
 // Splits the sequence of every (b, h) into chunks so that about `workgroups` workgroups exist.  The K/V pass
@@ -615,20 +616,41 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   __shared__ __align__(16) char s_q[kLinWaves][STRIP];       // wave-private Q strip
   __shared__ __align__(16) char otr[kLinWaves * SUB * OROW]; // wave-private output transpose buffers
 
-  const int BH = p.B * p.H;
-  const int bh = blockIdx.x % BH;
-  const int ch = blockIdx.x / BH;
-  const int b = bh / p.H, h = bh % p.H;
   const int lane = lane_id(), wave = wave_id();
   const int g = lane >> 5, n = lane & 31;
   char* ost = otr + wave * SUB * OROW;
   char* tq = s_q[wave];
 
+  // Two ways to share the work.  out_wave_heads: a workgroup takes four adjacent heads of one token chunk, one
+  // head per wave, every wave walking all strips of the chunk: with heads adjacent in memory the workgroup
+  // then reads and writes 512 contiguous bytes per token instead of 128 (the DRAM pages of a token row are
+  // touched by one workgroup at one time, not by sixteen at sixteen times).  Otherwise one head per
+  // workgroup, the strips of the chunk dealt round-robin to the waves.
+  int bh, ch, strip0, strip_step;
+  if (p.out_wave_heads) {
+    const int hq = p.H / kLinWaves, groups = p.B * hq;
+    const int bg = blockIdx.x % groups;
+    ch = blockIdx.x / groups;
+    bh = (bg / hq) * p.H + (bg % hq) * kLinWaves + wave;
+    strip0 = 0;
+    strip_step = 1;
+  } else {
+    const int BH = p.B * p.H;
+    bh = blockIdx.x % BH;
+    ch = blockIdx.x / BH;
+    strip0 = wave;
+    strip_step = kLinWaves;
+  }
+  const int b = bh / p.H, h = bh % p.H;
+
   const int tok_begin = ch * p.out_tiles_per_chunk * kLinTile;
   const int tok_end = min(p.S, tok_begin + p.out_tiles_per_chunk * kLinTile);
   const int nsub = (tok_end - tok_begin + SUB - 1) / SUB;
-  const int nmine = nsub > wave ? (nsub - wave + kLinWaves - 1) / kLinWaves : 0;
+  const int nmine = nsub > strip0 ? (nsub - strip0 + strip_step - 1) / strip_step : 0;
 
+  float winv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) winv[i] = p.winv[bh * 4 + i];
   // A operand: W^T[e][d], hi and lo, rows e = 32 eb + n, contraction slots d = 16 t + 8 g + [0..7]
   const uint16_t* w = p.w + (int64_t)bh * 2 * D * D;
   half8 whi[2][4], wlo[2][4];
@@ -643,9 +665,9 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   StripMover<SUB, kRowSwizzle> mvQ;
   mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
   uint4v rq[P][R];  // strips in flight, indexed by compile-time slot
-  auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * SUB; };
+  auto strip_row0 = [&](int i) { return tok_begin + (strip0 + strip_step * i) * SUB; };
   mvQ.limit_rows(nmine > 0 ? strip_row0(nmine - 1) + SUB - 1 : tok_begin);
-  __builtin_amdgcn_sched_barrier(0);  // W, then strip 0, then strip 1: loads complete in the order they are issued
+  __builtin_amdgcn_sched_barrier(0);  // scales and W, then strip 0, then strip 1: loads complete in the order they are issued
   mvQ.load(strip_row0(0), rq[0]);
   __builtin_amdgcn_sched_barrier(0);
   mvQ.load(strip_row0(1), rq[1]);
@@ -654,9 +676,6 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   // waits for the strip requested a few instructions earlier instead.
   static_assert(P * R == 8, "the wait below counts the loads of the two strips");
   __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8), every other counter at its maximum
-  float winv[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) winv[i] = p.winv[bh * 4 + i];
 
   char* obase = static_cast<char*>(p.o) + (b * p.so.b + h * p.so.h) * (int64_t)(F32OUT ? 4 : 2);
   const int64_t orow_bytes = p.so.s * (int64_t)(F32OUT ? 4 : 2);
@@ -802,6 +821,15 @@ hipError_t launch_linattn(const FtAttnArgs& a0, int kind, int normalize_q, int o
   lin_plan(a, kOutWorkgroups, &p.out_nch, &p.out_tiles_per_chunk);
   const bool ea = kind == FT_OP_EA;
   const bool nq = !ea && normalize_q;
+  // Four heads per workgroup in the output pass (see the kernel) where Q comes from HBM: B8 H16 S8192, EA
+  // 127.4 -> 121.2 us per call.  SimA with normalised queries has just read Q in its K/V pass and finds much of it
+  // in the memory-side cache; there the one-head form is the faster by 1 us (126.6 vs 127.7) and stays.
+  p.out_wave_heads = a.H % kLinWaves == 0 && !nq;
+  if (p.out_wave_heads) {  // the same number of workgroups over a quarter as many (b, head group) pairs
+    FtAttnArgs quarter = a;
+    quarter.H = a.H / kLinWaves;
+    lin_plan(quarter, kOutWorkgroups, &p.out_nch, &p.out_tiles_per_chunk);
+  }
   const bool f32 = out_dtype == FT_F32;
   const size_t bh = (size_t)a.B * a.H;
   char* base = static_cast<char*>(ws);
@@ -811,7 +839,7 @@ hipError_t launch_linattn(const FtAttnArgs& a0, int kind, int normalize_q, int o
   base += bh * 2 * kLinD * kLinD * sizeof(uint16_t);
   p.winv = reinterpret_cast<float*>(base);
 
-  const dim3 grid1((unsigned)(bh * p.nch)), grid3((unsigned)(bh * p.out_nch)), blk(kLinThreads);
+  const dim3 grid1((unsigned)(bh * p.nch)), grid3((unsigned)((p.out_wave_heads ? bh / kLinWaves : bh) * p.out_nch)), blk(kLinThreads);
   if (ea)
     hipLaunchKernelGGL((linattn_kv_kernel<true, false>), grid1, blk, 0, s, p);
   else if (nq)

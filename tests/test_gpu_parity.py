@@ -304,7 +304,9 @@ def test_builder_callables_have_reference_signatures(gpu):
 
 # ------------------------------------------------------------------ linear attention
 
-@pytest.mark.parametrize("B,S,H,seed", [(1, 128, 2, 0), (2, 200, 2, 1), (1, 1000, 3, 2), (1, 64, 1, 3), (1, 2500, 2, 4)])
+# (head counts that are multiples of four take the output pass's four-heads-per-workgroup form)
+@pytest.mark.parametrize("B,S,H,seed", [(1, 128, 2, 0), (2, 200, 2, 1), (1, 1000, 3, 2), (1, 64, 1, 3), (1, 2500, 2, 4),
+                                        (2, 200, 4, 5), (1, 1000, 8, 6), (1, 97, 4, 7)])
 def test_ea_sima_small(gpu, B, S, H, seed):
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, 64, seed=seed)
   check_o(ops.ea(qd, kd, vd), oracle.ea_forward(q, k, v))
@@ -316,9 +318,12 @@ def test_ea_sima_small(gpu, B, S, H, seed):
   o16 = ops.sima(qd, kd, vd)
   assert o16.dtype == torch.float16
   assert (o16.float().cpu() - ref32.half().float()).abs().max().item() <= max(6e-8, 1e-3 * ref32.abs().max().item())
+  # a [B,H,S,D] storage order (heads far apart in memory) is a strided view of the same kernels: same bits
+  qt, kt, vt = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (qd, kd, vd))
+  assert torch.equal(ops.ea(qt, kt, vt), ops.ea(qd, kd, vd))
 
 
-@pytest.mark.parametrize("B,S,H,seed", [(2, 200, 4, 20), (1, 333, 2, 21), (1, 784, 6, 22), (1, 1, 2, 23)])
+@pytest.mark.parametrize("B,S,H,seed", [(2, 200, 4, 20), (1, 333, 2, 21), (1, 784, 6, 22), (1, 1, 2, 23), (1, 300, 8, 24)])
 def test_ea_sima_head_dim_32(gpu, B, S, H, seed):
   """head_dim 32 (the literal shape of bench/ea.mlir:7-9) runs as pairs of adjacent heads on the 64-channel
   kernels; nothing of one head may leak into its neighbour."""
