@@ -129,3 +129,33 @@ def softcap_attention(q, k, v, cap):
       e = np.exp(s - s.max(axis=1, keepdims=True))
       O[b, :, h, :] = (e / e.sum(axis=1, keepdims=True)) @ v[b, :, h, :].astype(np.float64)
   return O
+
+
+def rounding_tie_slack(q, k, weights, tau=1.0, power=1, near=1e-3):
+  """How far a per-key score may move because QK^T values sit on fp16 rounding ties: [B,H,Skv], relative.
+
+  The reference rounds QK^T to fp16.  With fp16 inputs the exact dot product is often within 1e-4 ulp of the
+  midpoint of two fp16 values, and the order of the fp32 accumulation (torch's CPU matmul, an exact sum rounded
+  once, an MFMA) then decides which neighbour it becomes: every one of them is the reference's definition.  The
+  neighbour changes the logit by one fp16 ulp u of the raw product, the weight exp(logit / tau) of that pair by
+  d = exp(u / (sqrt(D) tau)) - 1, and through the row's normaliser every other weight of the row by w d, w being
+  the probability of the pair; a key whose column is dominated by such a row moves with it.
+  weights: [B,H,Sq,Skv] fp32, the row-normalised probabilities whose `power`-th powers sum down the columns to
+  the score."""
+  q, k = (t.numpy().astype(np.float64) for t in (q, k))
+  w = weights.numpy().astype(np.float64)
+  B, Sq, H, D = q.shape
+  out = np.zeros(w.shape[:2] + (w.shape[3],))
+  for b in range(B):
+    for h in range(H):
+      s = q[b, :, h, :] @ k[b, :, h, :].T                      # exact: fp16 products and their sums fit in fp64
+      r = s.astype(np.float16).astype(np.float64)              # the nearest fp16 value
+      sp = np.spacing(np.abs(r).astype(np.float16)).astype(np.float64)
+      dist = np.abs(np.abs(s - r) - sp / 2) / sp               # distance to the midpoint next to it, in ulps
+      d = np.where((dist < near) & (w[b, h] > 0), np.expm1(sp / (np.sqrt(D) * tau)), 0.0)
+      own = np.expm1(power * np.log1p(d))                      # the pair's own term
+      row = power * (w[b, h] * d).sum(axis=1, keepdims=True)   # every term of a row with a tie in it
+      wp = w[b, h] ** power
+      col = wp.sum(axis=0)
+      out[b, h] = (wp * (own + row)).sum(axis=0) / np.where(col > 0, col, 1.0)
+  return out
