@@ -36,6 +36,11 @@ struct F16 {
   static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  // 16x16x32: lane l holds row (A) / column (B) l % 16 and contraction slots 8 (l / 16) + [0..7]; of the result,
+  // column l % 16 and rows 4 (l / 16) + [0..3]
+  static __device__ __forceinline__ float4v mfma16(vec8 a, vec8 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
   static __device__ __forceinline__ uint16_t from_float(float x) {
     _Float16 h = (_Float16)x;
     return __builtin_bit_cast(uint16_t, h);
@@ -59,6 +64,9 @@ struct BF16 {
   static __device__ __forceinline__ elem to_elem(uint16_t bits) { return __builtin_bit_cast(__bf16, bits); }
   static __device__ __forceinline__ float16v mfma(vec8 a, vec8 b, float16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float4v mfma16(vec8 a, vec8 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ uint16_t from_float(float x) {  // round to nearest even (v_cvt_pk_bf16_f32)
     return __builtin_bit_cast(uint16_t, (__bf16)x);
