@@ -151,6 +151,27 @@ def test_scores_where_a_logit_sits_on_an_fp16_rounding_tie(gpu, B, S, kv, H, D, 
     check(s, w.sum(2), brute.rounding_tie_slack(q, k, w, tau=tau), f"keyformer tensor tau={tau}")
 
 
+@pytest.mark.parametrize("Skv", [15, 16, 17, 31, 33, 47, 49, 127, 129, 143, 145, 161])
+def test_column_sums_at_key_counts_around_the_block_edges(gpu, Skv):
+  """The column pass gives a lane two key columns 16 apart, a wave 32 and a workgroup 128: key counts one off
+  those edges, square and with three more keys than queries, both head sizes, against the oracle
+  (cases/kernels/roco.py:42-46, kf.py:36-40) and, for the seeded KeyFormer stream, the packed against the general path."""
+  for Sq, D, seed in ((Skv, 128, Skv), (max(1, Skv - 3), 64, 1000 + Skv)):
+    (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, Sq, 2, D, seed=seed, kv_len=None if Sq == Skv else Skv)
+    ref_o, r1, r2 = oracle.roco_forward(q, k, v)
+    out, s1, s2 = ops.roco(qd, kd, vd)
+    check_o(out, ref_o); check_score(s1, r1); check_score(s2, r2)
+    assert s1.shape == (1, 2, Skv)
+    es = oracle.seeded_exp_rand(seed, 1, 2, Sq, Skv)
+    _, ref_kf = oracle.keyformer_forward(q, k, v, es, tau=1.0)
+    check_score(ops.keyformer(qd, kd, vd, None, tau=1.0, seed=seed)[1], ref_kf)
+    _, ref_kf = oracle.keyformer_forward(q, k, v, es, tau=1.5)
+    check_score(ops.keyformer(qd, kd, vd, None, tau=1.5, seed=seed)[1], ref_kf)
+    check_score(ops.keyformer(qd, kd, vd, es.to(gpu), tau=1.5)[1], ref_kf)
+    if Sq == Skv:
+      check_corm(ops.corm(qd, kd, vd)[1], oracle.corm_margin(q, k, oracle.corm_mask_rule(Sq, Sq)))
+
+
 def test_rectangular_prefill_offset(gpu):
   # Sq < Skv: query i sees keys j <= i + (Skv - Sq)  (cases/kernels/attn.py:23)
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 96, 2, 128, seed=3, kv_len=232)
