@@ -24,8 +24,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 # HBM-side bytes per launch of the attention kernel at the benchmark shape, from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by the readings of a 256 MiB tensor copy in the same run (--calibrate-copy):
-# 78718 x 2 KiB read + 33280 x 1 KiB written (profiles/attn_colstats_h2o_s4096_pmc_traffic.txt)
-ATTN_TRAFFIC_BYTES = 195.29e6
+# 78704 x 2 KiB read + 33280 x 1 KiB written (profiles/attn_colstats_h2o_s4096_pmc_traffic.txt)
+ATTN_TRAFFIC_BYTES = 195.27e6
 
 
 KERNEL_TIMING_ITERS = 300    # timed launches of the kernel-alone and step event loops, whatever --steps says
