@@ -27,6 +27,9 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
          # registers, scratch and spills of every kernel, written next to its object (see _resources): a spilled
          # register in a loop that keeps direct-to-LDS loads in flight costs far more than its reload
          "-Rpass-analysis=kernel-resource-usage"]
+# The attention kernels take row maxima of MFMA results with plain fmaxf chains: without NaN honouring they become
+# v_max3_f32 with no quieting moves, and stay visible to the compiler's hazard handling (no kernel relies on NaNs)
+EXTRA_FLAGS = {src: ["-fno-honor-nans"] for src in ("attn_fwd_f16_d128.hip", "attn_fwd_f16_d64.hip", "attn_fwd_bf16_d128.hip", "attn_fwd_bf16_d64.hip")}
 
 
 def _hipcc():
@@ -67,7 +70,7 @@ def _compile(src, force):
   deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS]
   if not force and not _stale(obj, deps):
     return obj, ""
-  cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+  cmd = [_hipcc()] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
   res = subprocess.run(cmd, capture_output=True, text=True)
   if res.returncode != 0:
     raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")

@@ -284,10 +284,15 @@ static __device__ __align__(256) unsigned char scratch[FT_STATIC_SCRATCH_BYTES];
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];  // zero-initialised; a racing first call stores the same address twice
 
-int static_scratch(void** out) {
+int static_scratch(void** out, hipStream_t stream) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  // the buffer handed out is the current device's copy: a stream of another device would run the kernels there
+  // with this device's address
+  int sdev = dev;
+  if (stream && hipStreamGetDevice(stream, &sdev) == hipSuccess && sdev != dev)
+    return fail(FT_EINVAL, "stream belongs to device %d, the current device is %d", sdev, dev);
   if (dev < 0 || dev >= kMaxDevices) return fail(FT_EUNSUPPORTED, "device index %d beyond the %d this entry point tracks", dev, kMaxDevices);
   void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (!ptr) {
@@ -352,7 +357,7 @@ int ft_attn_colstats_fwd_static(const FtAttnArgs* a, float* colsum, float* colsu
     return fail(FT_EWORKSPACE, "problem needs %zu bytes of scratch, the static buffer holds %zu: use ft_attn_colstats_fwd with a workspace",
                 need, (size_t)FT_STATIC_SCRATCH_BYTES);
   void* ws = nullptr;
-  if (int rc = static_scratch(&ws)) return rc;
+  if (int rc = static_scratch(&ws, (hipStream_t)stream)) return rc;
   return run_colstats(a, colsum, colsumsq, ws, stream);
 }
 

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdlib>
 
 #include "kernel_params.h"
 
@@ -18,6 +19,21 @@ int device_cu_count() {
     cus[dev].store(n, std::memory_order_relaxed);
   }
   return n;
+}
+
+// Test hook: FT_ATTN_FORM in the environment overrides the launch shape the dispatcher would pick for the
+// problem size ("4": 128-row workgroups; "8": 256-row workgroups, one query block each; "8x2": 256-row workgroups
+// that take the heaviest and the lightest remaining block; an "h" appended: head-major workgroup order), so that
+// every form can be checked on every shape whatever the CU count of the device.  Read on every launch.
+int attn_form_override() {
+  const char* e = getenv("FT_ATTN_FORM");
+  if (!e || !*e) return 0;
+  int form = 0;
+  if (e[0] == '4') form = 1;
+  else if (e[0] == '8') form = (e[1] == 'x' && e[2] == '2') ? 3 : 2;
+  for (const char* c = e; *c; ++c)
+    if (*c == 'h') form |= 8;
+  return form;
 }
 
 hipError_t launch_attn_f16_d64(const AttnKernelParams& p, bool causal, bool emu, int kf, hipStream_t s);

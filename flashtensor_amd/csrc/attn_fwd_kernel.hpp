@@ -62,19 +62,28 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 
   const int BH = p.B * p.H;
   const int nMB = (p.Sq + BM - 1) / BM;
-  const int bh = blockIdx.x % BH;
+  // (b, h) pair and rank among that pair's workgroups.  Workgroups are dealt round-robin to the 8 XCDs and, inside
+  // an XCD, start in index order.  head_major: the workgroups of an XCD walk through that XCD's pairs one after
+  // the other (all ranks of a pair are neighbours in the XCD's order), so that the workgroups resident on an XCD
+  // at one time share the K/V of a few pairs in its L2; otherwise rank-major (every pair's rank 0 first).
+  int bh = blockIdx.x % BH, rank = blockIdx.x / BH;
+  if (p.head_major) {
+    const int li = blockIdx.x >> 3, nrank = gridDim.x / BH;
+    bh = (blockIdx.x & 7) + 8 * (li / nrank);
+    rank = li % nrank;
+  }
   // Heaviest (last) query blocks of every head first: longest-processing-time order keeps the causal
   // triangle balanced over the CUs.  Workgroups are dealt round-robin to the 8 XCDs, so with B*H a
   // multiple of 8 a head stays on one XCD and its K/V are shared through that XCD's L2.  (Walking an XCD
   // through its heads one at a time cuts the K/V re-reads from 1.6x to 1.1x of the operand size but
   // loses the balance: measured 15% slower.)
-  int mb = nMB - 1 - blockIdx.x / BH;
+  int mb = nMB - 1 - rank;
   if (p.pair_order) {
     // Every workgroup is resident from the start (no more of them than slots), so nothing is left to hand out
     // as CUs free up: the heavy half is dealt first, descending, then the light half ascending, which tends to
     // put a heavy and a light block on the same CU (measured 50 -> 47 us at B1 H32 S2048; with more
     // workgroups than slots the descending order wins: 144 vs 164 us at S4096).
-    const int rank = blockIdx.x / BH, half = (nMB + 1) / 2;
+    const int half = (nMB + 1) / 2;
     mb = rank < half ? nMB - 1 - rank : rank - half;
   }
   const int b = bh / p.H, h = bh % p.H;
@@ -86,9 +95,9 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // (compiled in only where the second pass costs no registers: with it the 4-wave form and the packed KeyFormer
   // modes spill, and a spilled register's reload waits for the tile loads in flight: both count in vmcnt)
   constexpr bool kTwoPass = WAVES == 8 && (KF == kKfNone || KF == kKfSoftcap);
-  const int npass = (kTwoPass && p.two_blocks && 2 * (int)(blockIdx.x / BH) != nMB - 1) ? 2 : 1;
+  const int npass = (kTwoPass && p.two_blocks && 2 * rank != nMB - 1) ? 2 : 1;
   for (int pass = 0; pass < npass; ++pass) {
-  if (kTwoPass && p.two_blocks) mb = pass == 0 ? nMB - 1 - (int)(blockIdx.x / BH) : (int)(blockIdx.x / BH);
+  if (kTwoPass && p.two_blocks) mb = pass == 0 ? nMB - 1 - rank : rank;
   if (pass) __syncthreads();  // every wave has left the first block's K/V tiles
   const int m0 = mb * BM;
   const int qi = m0 + wave * 32 + n;
@@ -232,8 +241,9 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
       const int jl = 32 * mbk + 8 * (r >> 2) + (r & 3);
       return jl > lim ? NEG_INF : s[mbk][r];
     };
-    // four independent chains, then a short tree: the reduction is latency-, not throughput-bound.  Only
-    // three-operand maxima: a two-operand fmaxf on MFMA results costs two extra NaN-quieting moves.
+    // four independent chains, then a short tree: the reduction is latency-, not throughput-bound.  Three-operand
+    // maxima throughout (v_max3_f32; this translation unit is built without NaN honouring, so none of them is
+    // preceded by quieting moves of the MFMA results).
     float m4[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -543,11 +553,8 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // ---- mask-free tiles, two per trip so that the two score buffers swap roles without copies
   // pairs (it, it+1) of mask-free tiles whose staged tiles K[it+2], K[it+3], V[it+1], V[it+2] are whole tiles
   const int nf2 = max(0, min(n_fast, p.Skv / BN - 2)) & ~1;
-  // tiles from nf2 on go through the masked instance (which is exact for a tile that needs no mask as well).
-  // Tile 0 always does: its maximum directly follows the MFMAs that produce the scores, and the mask-free instance
-  // reads them with hand-written v_max3 instructions, for which the compiler does not insert the wait states a
-  // vector instruction needs after the matrix instruction whose result it reads (in the loop sixteen PV MFMAs
-  // lie between the two); the masked instance reads them through ordinary selects first.
+  // tiles from nf2 on go through the masked instance (which is exact for a tile that needs no mask as well); so
+  // does tile 0, which may be one of them.
   pend_max = tile_max(std::true_type{}, S0, 0);
   for (; it < nf2 - 2; it += 2) {
     wait_vmem();
@@ -705,33 +712,41 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 // ---------------------------------------------------------------------------------------------------
 // launch-shape selection (host)
 
-int device_cu_count();  // attn_fwd.hip
+int device_cu_count();     // attn_fwd.hip
+int attn_form_override();  // attn_fwd.hip: 0, or (1: 4 waves, 2: 8 waves, 3: 8 waves and two blocks) | 8: head-major order
 
 template <typename T, int D, bool CAUSAL, bool EMU, int KF>
 hipError_t launch_one(const AttnKernelParams& p0, hipStream_t stream) {
   AttnKernelParams p = p0;
   p.pair_order = 0;
+  p.two_blocks = 0;
+  p.head_major = 0;
+  const int forced = attn_form_override();
+  const int64_t BH = (int64_t)p.B * p.H;
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
   // there are half as many of them: used on the pipelined paths once they still fill the chip twice
   constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast;
-  p.two_blocks = 0;
   if constexpr (kHas8) {
     const int nMB8 = (p.Sq + 255) / 256;
-    const int64_t n8 = (int64_t)nMB8 * p.B * p.H;
+    const int64_t n8 = (int64_t)nMB8 * BH;
     const int64_t cus = device_cu_count();
-    if (n8 >= 2 * cus) {
+    if ((forced & 7) ? (forced & 7) >= 2 : n8 >= 2 * cus) {
       // causal: pair the heaviest block with the lightest inside one workgroup when the pairs come out as whole
       // rounds of the chip (or as many rounds that a ragged last one does not matter)
-      const int64_t pairs = (int64_t)((nMB8 + 1) / 2) * p.B * p.H;
-      p.two_blocks = kAttnTwoBlocks && (KF == kKfNone || KF == kKfSoftcap) && CAUSAL && nMB8 >= 2 && (pairs % cus == 0 || pairs >= 8 * cus);
+      const int64_t pairs = (int64_t)((nMB8 + 1) / 2) * BH;
+      constexpr bool kCanPair = kAttnTwoBlocks && (KF == kKfNone || KF == kKfSoftcap) && CAUSAL;
+      p.two_blocks = kCanPair && nMB8 >= 2 && ((forced & 7) ? (forced & 7) == 3 : (pairs % cus == 0 || pairs >= 8 * cus));
       const int64_t grid = p.two_blocks ? pairs : n8;
+      // equal workgroups in several rounds: let an XCD finish a pair's blocks before it starts the next pair's
+      p.head_major = BH % 8 == 0 && (forced ? (forced & 8) != 0 : (p.two_blocks && grid >= 3 * cus));
       hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 8>), dim3((unsigned)grid), dim3(512), 0, stream, p);
       return hipGetLastError();
     }
   }
   const int nMB = (p.Sq + 127) / 128;
-  dim3 grid((unsigned)(nMB * p.B * p.H));
+  dim3 grid((unsigned)(nMB * BH));
   p.pair_order = CAUSAL && (int64_t)grid.x <= 2 * (int64_t)device_cu_count();  // two workgroups of this form per CU
+  p.head_major = BH % 8 == 0 && (forced & 8) != 0 && !p.pair_order;
   hipLaunchKernelGGL((attn_fwd_kernel<T, D, CAUSAL, EMU, KF, 4>), grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }

@@ -56,12 +56,17 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, CAUSA
   // one LDS object per buffer: reads of one do not wait for the direct-to-LDS loads in flight into the other
   __shared__ __align__(16) char ldsQ0[TILE_BYTES];
   __shared__ __align__(16) char ldsQ1[TILE_BYTES];
+  __shared__ __align__(16) char ldsQ2[TILE_BYTES];  // tile t lives in buffer t % 3: two tiles in flight behind the one being read
   __shared__ __align__(16) float ldsLse[2 * BQ];     // row normalisers of the current / next tile
   __shared__ __align__(16) uint32_t ldsRow[2 * BQ];  // noise row terms (seeded KeyFormer)
 
   const int BH = p.B * p.H;
+  // Low key blocks see the most rows under the causal mask: heaviest first, every (b, h) pair's block 0 before any
+  // pair's block 1.  (Letting an XCD finish one pair's blocks before the next pair's, which pays in the attention
+  // pass, loses that balance here: measured 974 against 955 us for the B4 H32 S4096 sum-of-squares call, 267
+  // against 239 us at B1.)
   const int bh = blockIdx.x % BH;
-  const int jb = blockIdx.x / BH;  // low key blocks see the most rows under the causal mask: heaviest first
+  const int jb = blockIdx.x / BH;
   const int b = bh / p.H, h = bh % p.H;
   const int j0 = jb * BK;
   const int lane = lane_id(), wave = wave_id();
@@ -414,18 +419,39 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, CAUSA
   };
   STile S0;
   if (ntiles > 0) {
-    // ---- prologue: Q[0], Q[1] in flight; rows of tile 0; scores of tile 0
+    // ---- prologue: Q[0], Q[1], Q[2] in flight; rows of tile 0; scores of tile 0
     if (kTensor) load_er(er, 0);
     stage_q(0, ldsQ0);
     stage_q(1, ldsQ1);
+    stage_q(2, ldsQ2);
     store_rows(0, load_rows(0));
     float lse_next = load_rows(1);  // rows of the tile after the current one, in flight
     wait_vmem();
     __syncthreads();
     qk(S0, ldsQ0);
 
-    // One iteration = one barrier.  On entry Q[t+1] has been requested and S0 holds the scores of
-    // tile t; Q[t+2] is requested into the buffer whose tile was consumed one iteration ago.
+    // One iteration = one barrier.  On entry to iteration t, S0 holds the scores of tile t, Q[t+1] (read in this
+    // iteration) and Q[t+2] have been requested; Q[t+3] is requested into the buffer of tile t.  The wait at the
+    // top is for Q[t+1] only: loads complete in order, and the staging loads of Q[t+2] (kStageLoads per thread, the
+    // newest in flight) may stay outstanding.  The row normalisers of tile t+2 are fetched before those staging
+    // loads, so that waiting for them does not wait for the tile.
+    constexpr int kStageLoads = BQ * G::CPR / NT;
+    static_assert(kStageLoads == 4 || kStageLoads == 2, "s_waitcnt immediates below");
+    auto wait_tile = [&](int t) __attribute__((always_inline)) {
+      if (!kTensor && t + 2 < ntiles) {
+        // vmcnt(kStageLoads) lgkmcnt(0); a bare barrier: __syncthreads() carries a fence that drains every load
+        __builtin_amdgcn_s_waitcnt(kStageLoads == 4 ? 0x0074 : 0x0072);
+        __builtin_amdgcn_s_barrier();
+      } else {
+        wait_vmem();
+        __syncthreads();
+      }
+    };
+    char *b0 = ldsQ0, *b1 = ldsQ1, *b2 = ldsQ2;  // buffers of tiles t, t + 1, t + 2
+    auto rotate = [&]() __attribute__((always_inline)) {
+      char* f = b0;
+      b0 = b1, b1 = b2, b2 = f;
+    };
     auto take_next_er = [&]() {
       // nothing of the tile may be scheduled below this point: the wait for the prefetched slice (which, loads
       // completing in order, is also a wait for the Q tile queued behind it) belongs at the very end
@@ -437,61 +463,65 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, CAUSA
     };
     int t = 0;
     for (; t < n_masked; ++t) {
-      wait_vmem();
-      __syncthreads();
+      wait_tile(t);
       if (kTensor) load_er(er_nx, t + 1);  // ahead of the staging loads: waiting for it does not wait for them
-      stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
       store_rows(t + 1, lse_next);
       lse_next = load_rows(t + 2);
+      stage_q(t + 3, b0);
       // every row of this tile above the diagonal for all 32 keys of the wave: nothing to add
       const bool skip = CAUSAL && (wave_key0 > i_begin + t * BQ + BQ - 1 + p.off);
       if (!skip) reduce_tile(std::true_type{}, S0, t);
-      qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
+      qk(S0, b1);
       if (kTensor) take_next_er();
+      rotate();
     }
     // Tensor modes are bound by the HBM stream of the tensor: one tile per trip, the registers of the second
     // score buffer hold the prefetched slice instead.
     if (kTensor) {
       for (; t < ntiles; ++t) {
-        wait_vmem();
-        __syncthreads();
+        wait_tile(t);
         load_er(er_nx, t + 1);
-        stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
         store_rows(t + 1, lse_next);
         lse_next = load_rows(t + 2);
+        stage_q(t + 3, b0);
         reduce_tile(std::false_type{}, S0, t);
-        qk(S0, (t & 1) ? ldsQ0 : ldsQ1);
+        qk(S0, b1);
         take_next_er();
+        rotate();
       }
     }
-    // mask-free tiles (the tensor modes have none left here), two per trip so that each half names its LDS
-    // buffers once
+    // mask-free tiles (the tensor modes have none left here)
     if constexpr (k16) {
-      if ((ntiles - t) & 1) {  // make the remainder even with one single step
-        wait_vmem();
-        __syncthreads();
-        stage_q(t + 2, (t & 1) ? ldsQ1 : ldsQ0);
-        store_rows(t + 1, lse_next);
-        lse_next = load_rows(t + 2);
-        reduce_qk(S0, (t & 1) ? ldsQ0 : ldsQ1, t);
-        ++t;
+      // While tile t + 3 is a whole tile every load of an iteration is issued unconditionally, so that the waits
+      // can be counted: kStageLoads staging loads (Q[t+2]) stay in flight across the barrier.  A clean start
+      // (nothing outstanding) keeps the compiler's own wait for the row normalisers at that count as well.
+      const int nfull = (p.Sq - i_begin) / BQ;  // whole tiles
+      if (t + 3 < nfull) wait_vmem();
+      for (; t + 3 < nfull; ++t) {
+        // vmcnt(kStageLoads) lgkmcnt(0), then a bare barrier: __syncthreads() carries a fence that drains every load
+        __builtin_amdgcn_s_waitcnt(kStageLoads == 4 ? 0x0074 : 0x0072);
+        __builtin_amdgcn_s_barrier();
+        if (threadIdx.x < BQ) {
+          const int i = i_begin + (t + 1) * BQ + threadIdx.x;
+          float nl = -lse_next;
+          if (MODE == kStatCormRule) nl += __builtin_amdgcn_logf((float)(i + 1));
+          if (MODE == kStatKfSeededFast) nl -= kLog2Ln2 * p.inv_tau;
+          ldsLse[((t + 1) & 1) * BQ + threadIdx.x] = nl;
+          if (kSeeded) ldsRow[((t + 1) & 1) * BQ + threadIdx.x] = noise_row(nk, (uint32_t)i);
+        }
+        lse_next = lse_bh[i_begin + (t + 2) * BQ + (threadIdx.x & (BQ - 1))];
+        __builtin_amdgcn_sched_barrier(0);  // the normalisers first: their wait must not reach into the staging loads
+        stQ.issue_full(i_begin + (t + 3) * BQ, b0);
+        reduce_qk(S0, b1, t);
+        rotate();
       }
-      const bool odd = t & 1;  // parity of the first tile of every pair
-      char* qa_buf = odd ? ldsQ1 : ldsQ0;  // holds tile t (consumed), refilled with t + 2
-      char* qb_buf = odd ? ldsQ0 : ldsQ1;  // holds tile t + 1
-      for (; t < ntiles; t += 2) {
-        wait_vmem();
-        __syncthreads();
-        stage_q(t + 2, qa_buf);
+      for (; t < ntiles; ++t) {
+        wait_tile(t);
         store_rows(t + 1, lse_next);
         lse_next = load_rows(t + 2);
-        reduce_qk(S0, qb_buf, t);
-        wait_vmem();
-        __syncthreads();
-        stage_q(t + 3, qb_buf);
-        store_rows(t + 2, lse_next);
-        lse_next = load_rows(t + 3);
-        reduce_qk(S0, qa_buf, t + 1);  // scores of tile t + 2: past the last tile they come from stale LDS and are discarded
+        stage_q(t + 3, b0);
+        reduce_qk(S0, b1, t);  // scores of tile t + 1: past the last tile they come from stale LDS and are discarded
+        rotate();
       }
     }
   }

@@ -102,12 +102,11 @@ __device__ __forceinline__ float xchg32(float x) {
 #endif
 }
 
-// max of three without the NaN-quieting moves the compiler adds around fmaxf on MFMA results
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
+// max of three, written so that the compiler sees it: it then inserts the wait states a vector instruction needs
+// after the matrix instruction whose result it reads (it inserts none around inline assembly).  Selected as
+// v_max3_f32 only in translation units built with -fno-honor-nans (the attention kernels): otherwise every fmaxf on
+// an MFMA result costs a NaN-quieting move per operand.
+__device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 
 // tanh to fp32 accuracy without a hardware instruction: odd polynomial where 1 - 2 / (e^2y + 1) would
 // cancel (|y| < 0.25, truncation error < 4e-7 relative), the exponential form elsewhere.

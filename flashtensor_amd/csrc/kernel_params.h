@@ -32,6 +32,7 @@ struct AttnKernelParams {
   int pair_order;   // block order of the causal attention kernel: heavy half descending, light half ascending
   int group;        // query heads per k/v head: query head h reads k/v head h / group
   int two_blocks;   // 256-row form: a workgroup takes query blocks nMB - 1 - slot and slot (set by the launcher)
+  int head_major;   // workgroup order inside an XCD: all blocks of a (b, h) pair before the next pair's (launcher)
 };
 
 struct ColstatsKernelParams {

@@ -99,7 +99,9 @@ int ft_attn_colstats_fwd(const FtAttnArgs* a, float* colsum, float* colsumsq, vo
  * carries on every GPU it is loaded on.  No counterpart in the reference.  Problems whose
  * ft_workspace_bytes(FT_OP_COLSTATS, a) exceeds the buffer are refused with FT_EWORKSPACE.  Calls no allocator.
  * All calls on one GPU share that GPU's buffer: two calls that overlap in time on one GPU (different streams or
- * threads) race; calls on one stream are ordered.  Results are those of ft_attn_colstats_fwd, bit for bit. */
+ * threads) race; calls on one stream are ordered.  Results are those of ft_attn_colstats_fwd, bit for bit.
+ * The buffer's address is looked up (hipGetSymbolAddress) on the first call on each device: make that first call
+ * outside graph capture.  `stream` must belong to the current device (FT_EINVAL otherwise). */
 #define FT_STATIC_SCRATCH_BYTES (8u << 20)
 int ft_attn_colstats_fwd_static(const FtAttnArgs* a, float* colsum, float* colsumsq, void* stream);
 

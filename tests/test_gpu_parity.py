@@ -670,6 +670,39 @@ def test_large_ragged_shapes_256_row_blocks(gpu, S, Skv, D, causal, seed):
     check_score(kf[:, :HS], oracle.keyformer_forward(*sub, es, tau=1.0)[1])
 
 
+@pytest.mark.parametrize("S,Skv,D,seed", [(4000, 4000, 128, 70), (3840, 3840, 128, 71), (3900, 4030, 128, 72), (3333, 3333, 64, 73),
+                                          (520, 520, 128, 74), (256, 300, 64, 75)])
+def test_every_launch_form_of_the_attention_pass_on_ragged_shapes(gpu, monkeypatch, S, Skv, D, seed):
+  """The dispatcher picks the workgroup form (128 rows; 256 rows; 256 rows taking the heaviest and the lightest
+  remaining block; head-major order) from the problem size and the CU count, so a given shape exercises one form
+  only on a given device.  FT_ATTN_FORM forces each in turn: ragged last blocks, an odd number of 256-row
+  blocks (the unpaired middle block), Skv > Sq, D = 64.  A wave works on the same 32 rows with the same tiles in
+  every form, so the outputs must agree bit for bit; one form is checked against the oracle."""
+  H = 8
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, D, seed=seed, kv_len=Skv)
+  res = {}
+  for form in ("4", "4h", "8", "8h", "8x2", "8x2h"):
+    monkeypatch.setenv("FT_ATTN_FORM", form)
+    out, s1 = ops.h2o(qd, kd, vd)
+    res[form] = (out, s1)
+    if D == 128:
+      res[form] += (ops.gemma2(qd, kd, vd),)
+  monkeypatch.delenv("FT_ATTN_FORM")
+  auto = ops.h2o(qd, kd, vd)
+  for form, r in res.items():
+    for a, b in zip(r, res["4"]):
+      assert torch.equal(a, b), form
+  assert torch.equal(auto[0], res["4"][0]) and torch.equal(auto[1], res["4"][1])
+  sub = tuple(t[:, :, :2].contiguous() for t in (q, k, v))
+  ref_o, ref_s = oracle.h2o_forward(*sub)
+  check_o(res["8x2"][0][:, :, :2], ref_o)
+  n_rows = (S - (torch.arange(Skv) - (Skv - S)).clamp_min(0)).float()
+  err = (res["8x2"][1][:, :2].float().cpu() - ref_s).abs() / ref_s.abs().clamp_min(1e-30)
+  assert (err <= 1e-3 + 4e-3 / n_rows).all(), f"score rel {err.max().item()}"   # as in the test above
+  if D == 128:
+    check_o(res["8x2"][2][:, :, :2], oracle.gemma2_forward(*sub))
+
+
 # ------------------------------------------------------------------ grouped queries, 2-D harness form
 
 @pytest.mark.parametrize("S,Skv,H,Hkv,D,masked", [(128, 128, 4, 2, 128, True), (200, 200, 8, 2, 64, True), (96, 232, 4, 1, 128, True),

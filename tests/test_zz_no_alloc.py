@@ -61,6 +61,40 @@ def test_static_scratch_entry_point_matches_the_workspace_one(gpu):
   assert torch.equal(ref[0], got[0]) and torch.equal(ref[1], got[1]) and got[1].shape == (1, 2, 264)
 
 
+def test_static_scratch_entry_point_at_the_benchmarked_shape_and_under_graph_capture(gpu):
+  """B1 H32 S4096 D128 (512 KB of normalisers, the 256-row two-block launch) bit for bit against the workspace entry
+  point; then the same call recorded into a HIP graph (after the eager call above has looked the buffer up) and
+  replayed on new inputs, with eager work between the replays."""
+  lib = _lib.load()
+  (q, k, v), (ref, got) = _call_both(lib, gpu, 1, 4096, 32, 128, 0, True)
+  for r, g in zip(ref, got):
+    assert torch.isfinite(g).all() and torch.equal(r, g)
+  assert torch.allclose(got[1].sum(-1).cpu(), torch.full((1, 32), 4096.0), rtol=1e-4)
+  B, S, H, D = 1, 600, 4, 128
+  qd, kd, vd = (torch.zeros(B, S, H, D, dtype=torch.float16, device=gpu) for _ in range(3))
+  out = torch.empty_like(qd)
+  s1 = torch.empty(B, H, S, dtype=torch.float32, device=gpu)
+  a = FtAttnArgs(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), _strides(qd), _strides(kd), _strides(vd),
+                 _strides(out), B, H, S, S, D, _lib.FT_F16, _lib.FT_CAUSAL, H)
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    stream = ctypes.c_void_p(torch.cuda.current_stream(gpu).cuda_stream)
+    assert lib.ft_attn_colstats_fwd_static(ctypes.byref(a), s1.data_ptr(), None, stream) == _lib.FT_OK, lib.ft_last_error().decode()
+  for seed in (41, 42, 43):
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed)
+    for dst, src in zip((qd, kd, vd), (q, k, v)):
+      dst.copy_(src.to(gpu))
+    graph.replay()
+    torch.cuda.synchronize()
+    got_o, got_s = out.clone(), s1.clone()
+    nbytes = lib.ft_workspace_bytes(_lib.FT_OP_COLSTATS, ctypes.byref(a))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=gpu)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(gpu).cuda_stream)
+    assert lib.ft_attn_colstats_fwd(ctypes.byref(a), s1.data_ptr(), None, ws.data_ptr(), nbytes, stream) == _lib.FT_OK
+    torch.cuda.synchronize()
+    assert torch.equal(got_o, out) and torch.equal(got_s, s1)
+
+
 def test_static_scratch_entry_point_limits_and_argument_checks(gpu):
   lib = _lib.load()
   limit = 8 << 20
