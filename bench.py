@@ -22,10 +22,21 @@ if ROOT not in sys.path:
 PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM-side bytes per launch of the attention kernel at the benchmark shape, from two rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE) scaled by the readings of a 256 MiB tensor copy in the same run (--calibrate-copy):
-# 78704 x 2 KiB read + 33280 x 1 KiB written (profiles/attn_colstats_h2o_s4096_pmc_traffic.txt)
-ATTN_TRAFFIC_BYTES = 195.27e6
+# HBM-side bytes per launch of the attention kernel at the benchmark shape come from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE, scaled by the readings of a 256 MiB tensor copy in the same run: --calibrate-copy).  They
+# cannot be measured from inside this process, so the line quotes the last measurement, kept with the commit it
+# was taken at in profiles/traffic.json, and says which commit that was.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(kernel):
+  """(HBM bytes per launch, the commit the counters were read at) for `kernel`, or (None, None)."""
+  try:
+    with open(TRAFFIC_FILE) as f:
+      entry = json.load(f)[kernel]
+    return float(entry["fetch_bytes"]) + float(entry["write_bytes"]), entry["measured_at_commit"]
+  except (OSError, KeyError, ValueError):
+    return None, None
 
 
 KERNEL_TIMING_ITERS = 300    # timed launches of the kernel-alone and step event loops, whatever --steps says
@@ -87,7 +98,7 @@ def per_config_table(dev, only=None, iters=100):
   def qkv(B, S, H, D):
     return tuple(torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3))
 
-  def add(name, shape, fn, flops, nbytes):
+  def add(name, shape, fn, flops, nbytes, split=False):
     if only is not None and only not in name:
       return
     try:
@@ -98,23 +109,28 @@ def per_config_table(dev, only=None, iters=100):
     tf, gb = flops / us / 1e6, nbytes / us / 1e3
     rows.append({"config": name, "shape": shape, "us": round(us, 1), "tflops": round(tf, 1),
                  "mfma_frac": round(tf / PEAK_MFMA_TFLOPS, 4), "gbs": round(gb, 1), "hbm_frac": round(gb / PEAK_HBM_GBS, 4)})
+    if split:
+      rows[-1]["kernels_us"] = kernel_split(fn)
 
-  def softmax_case(name, B, S, H, D, fn_of, extra_bytes=0):
+  def softmax_case(name, B, S, H, D, fn_of, extra_bytes=0, split=False):
     q, k, v = qkv(B, S, H, D)
-    add(name, f"B{B} H{H} S{S} D{D}", fn_of(q, k, v), 2.0 * B * H * S * S * D, 4.0 * B * S * H * D * 2 + extra_bytes)
+    add(name, f"B{B} H{H} S{S} D{D}", fn_of(q, k, v), 2.0 * B * H * S * S * D, 4.0 * B * S * H * D * 2 + extra_bytes, split)
 
   softmax_case("1 attn", 1, 1024, 32, 128, lambda q, k, v: (lambda: ops.attn(q, k, v)))
   softmax_case("2 h2o+topk", 1, 2048, 32, 128,
                lambda q, k, v: (lambda: ops.topk(ops.h2o(q, k, v)[1], 256)), extra_bytes=32 * 2048 * 4)
   softmax_case("2' h2o", 1, 4096, 32, 128, lambda q, k, v: (lambda: ops.h2o(q, k, v)), extra_bytes=32 * 4096 * 4)
+  # what reproducing the reference's fp16 rounding of the logits costs: the same call with the logits kept in fp32
+  softmax_case("2' h2o, logits in fp32 (FT_FAST_LOGITS)", 1, 4096, 32, 128,
+               lambda q, k, v: (lambda: ops.h2o(q, k, v, fast_logits=True)), extra_bytes=32 * 4096 * 4, split=True)
   softmax_case("3 keyformer seeded tau=1", 1, 4096, 32, 128,
-               lambda q, k, v: (lambda: ops.keyformer(q, k, v, None, tau=1.0, seed=1)), extra_bytes=32 * 4096 * 4)
+               lambda q, k, v: (lambda: ops.keyformer(q, k, v, None, tau=1.0, seed=1)), extra_bytes=32 * 4096 * 4, split=True)
   if only is None or only in "3t keyformer tensor noise tau=1.5":
     er = 1 + torch.randn(1, 32, 4096, 4096, dtype=torch.float32, device=dev).abs()
     softmax_case("3t keyformer tensor noise tau=1.5", 1, 4096, 32, 128,
                  lambda q, k, v: (lambda: ops.keyformer(q, k, v, er, tau=1.5)),
                  # both passes read the visible (lower-triangular) half of the noise tensor, nothing above the diagonal
-                 extra_bytes=2 * 32 * (4096 * 4097 // 2) * 4)
+                 extra_bytes=2 * 32 * (4096 * 4097 // 2) * 4, split=True)
     del er
   softmax_case("4 roco", 4, 4096, 32, 128, lambda q, k, v: (lambda: ops.roco(q, k, v)), extra_bytes=2 * 4 * 32 * 4096 * 4)
   # the other cases of the reference's zoo at their prepare() defaults (B=1 H=32 S=4096 D=128)
@@ -127,8 +143,8 @@ def per_config_table(dev, only=None, iters=100):
       (2 * q.numel() + 2 * kg.numel()) * 2.0 + 8 * 4096 * 4)
   q, k, v = qkv(8, 8192, 16, 64)
   lin_flops, lin_bytes = 2 * 2.0 * 8 * 16 * 8192 * 64 * 64, 4.0 * 8 * 16 * 8192 * 64 * 2
-  add("5 ea", "B8 H16 S8192 D64", lambda: ops.ea(q, k, v), lin_flops, lin_bytes)
-  add("5 sima", "B8 H16 S8192 D64", lambda: ops.sima(q, k, v), lin_flops, lin_bytes)
+  add("5 ea", "B8 H16 S8192 D64", lambda: ops.ea(q, k, v), lin_flops, lin_bytes, split=True)
+  add("5 sima", "B8 H16 S8192 D64", lambda: ops.sima(q, k, v), lin_flops, lin_bytes, split=True)
   del q, k, v
   # the whole function of bench/ea.mlir / bench/sima.mlir: hipBLASLt projections around the core (C = 1024)
   C, M = 16 * 64, 8 * 8192
@@ -150,6 +166,34 @@ def per_config_table(dev, only=None, iters=100):
   add("5c ea block, .mlir shape", "B64 S784 C128 H4 D32", lambda: ops.ea_block(x, wq, bq, wo, bo, 4),
       2 * 2.0 * 64 * 4 * 784 * 32 * 32 + 2.0 * M * 4 * C * C, (2.0 * M * C + 4 * C * C + 4 * C) * 2)
   return rows
+
+
+def kernel_split(fn, iters=20):
+  """Average device time per kernel name over `iters` calls of fn, from torch's profiler (kernel activity records):
+  which launch of a multi-launch call the time goes to.  Diagnostic: returns an error entry where the profiler is
+  not usable (another tracer attached, say)."""
+  import torch
+  try:
+    from torch.profiler import ProfilerActivity, profile
+    for _ in range(5):
+      fn()
+    torch.cuda.synchronize()
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+      for _ in range(iters):
+        fn()
+      torch.cuda.synchronize()
+    out = {}
+    for ev in prof.key_averages():
+      name, total = ev.key, getattr(ev, "device_time_total", None)
+      if total is None:
+        total = getattr(ev, "cuda_time_total", 0.0)
+      if "ft::" not in name or not total:
+        continue
+      short = name.split("ft::", 1)[1].split("<", 1)[0].split("(", 1)[0]
+      out[short] = round(out.get(short, 0.0) + total / iters, 1)
+    return out or {"error": "no kernel records"}
+  except Exception as e:
+    return {"error": f"{type(e).__name__}: {e}"}
 
 
 def mfma_probe(dev):
@@ -223,6 +267,8 @@ def main():
   torch.manual_seed(0)
 
   B, H, S, D = 1, 32, 4096, 128
+  # the CPU leg first, so that the GPU legs run back to back until the line is printed
+  cpu = None if args.no_cpu else cpu_baseline(B, S, H, D, args.cpu_heads)
   q, k, v = (torch.randn(B, S, H, D, dtype=torch.float16, device=dev) for _ in range(3))
   flops = 2.0 * B * H * S * S * D
   alg_bytes = 4.0 * B * S * H * D * 2 + B * H * S * 4
@@ -266,6 +312,7 @@ def main():
   cold_us = event_time_us(cold_step)
   del sets
 
+  traffic, traffic_commit = measured_traffic("attn_fwd_kernel")
   result = {
       "metric": "fused attn+score (H2O) algorithmic TFLOP/s at S=4096, 1 GPU",
       "value": round(flops / dt / 1e12, 2),
@@ -287,7 +334,8 @@ def main():
       "frac_of_fp16_mfma_peak": round(flops / dt / 1e12 / PEAK_MFMA_TFLOPS, 4),
       "algorithmic_gbs": round(alg_bytes / dt / 1e9, 1),
       "roofline": {"bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(attn_tflops, 1), "peak": PEAK_MFMA_TFLOPS,
-                   "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_MFMA_TFLOPS, 4), "traffic": ATTN_TRAFFIC_BYTES,
+                   "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_MFMA_TFLOPS, 4), "traffic": traffic,
+                   "traffic_measured_at": traffic_commit,
                    "us_per_launch": round(attn_us, 1), "algorithmic_flop_per_launch": flops,
                    "timed_launches": KERNEL_TIMING_ITERS},
       "kernels_us": {"attn_fwd_kernel": round(attn_us, 1), "colstats_kernel": round(step_us - attn_us, 1),
@@ -300,10 +348,7 @@ def main():
     result["mfma_probe"] = {"error": f"{type(e).__name__}: {e}"}
   if not args.no_configs:
     result["per_config"] = per_config_table(dev, args.only, args.config_iters)
-  if not args.no_cpu:
-    result["cpu_baseline"] = cpu_baseline(B, S, H, D, args.cpu_heads)
-  else:
-    result["cpu_baseline"] = None
+  result["cpu_baseline"] = cpu
   print(json.dumps(result))
 
 

@@ -392,6 +392,10 @@ int ft_keyformer_fwd(const FtAttnArgs* a, const FtNoise* noise, float tau, float
   // seeded noise, fp16, reference rounding: the packed path (tau == 1 needs 1 / E only; tau >= 0.25 keeps
   // the perturbed sum inside fp32 range under the plain softmax's stabiliser); otherwise the generic path
   int amode = tensor ? ft::kKfTensor : ft::kKfSeeded, cmode = tensor ? ft::kStatKfTensor : ft::kStatKfSeeded;
+  // noise rows that can be fetched in 16-byte chunks through a buffer descriptor of the (b, h) slice: the attention
+  // pass lands them in LDS a tile ahead
+  if (tensor && p.er_vec4 && a->Skv % 4 == 0 && (int64_t)a->Sq * noise->stride_row * 4 < (int64_t)0x7fffffff)
+    amode = ft::kKfTensorLds;
   if (!tensor && emu && a->dtype == FT_F16) {
     if (tau == 1.f) {
       amode = ft::kKfSeededTau1;

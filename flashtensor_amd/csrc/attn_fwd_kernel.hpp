@@ -34,7 +34,7 @@ constexpr bool kAttnTwoBlocks = true;
 constexpr float kRescaleSlack = 6.f;
 
 template <typename T, int D, bool CAUSAL, bool EMU, int KF, int WAVES>
-__global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const AttnKernelParams p) {
+__global__ void __launch_bounds__(64 * WAVES, (KF == kKfTensorLds ? 1 : 8 / WAVES)) attn_fwd_kernel(const AttnKernelParams p) {
   constexpr int BM = 32 * WAVES, BN = kAttnBN, NT = 64 * WAVES;
   constexpr int KSTEPS = D / 16;
   constexpr int DB = D / 32;
@@ -48,6 +48,8 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   // logits, and the packed seeded KeyFormer modes (fp16)
   constexpr bool kFastMasked = (kIsF16 && EMU && kKfFast) || KF == kKfNone || KF == kKfSoftcap;
   constexpr bool kCap = KF == kKfSoftcap;
+  constexpr bool kErLds = KF == kKfTensorLds;               // noise tensor staged through LDS
+  constexpr bool kTensor = KF == kKfTensor || kErLds;
   static_assert(!kKfFast || (kIsF16 && EMU), "the packed KeyFormer modes exist for fp16 with reference rounding only");
   // Software pipeline across tiles: the QK^T MFMAs of tile it+1 are issued in the same iteration as the
   // softmax (VALU) and PV MFMAs of tile it, so the matrix and vector pipes overlap inside one wave.
@@ -59,6 +61,10 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
   __shared__ __align__(16) char ldsV0[TILE_BYTES];
   __shared__ __align__(16) char ldsV1[TILE_BYTES];
   __shared__ __align__(16) uint32_t ldsCol[2 * BN];  // noise column terms of the current / next tile
+  // kKfTensorLds: every wave's slice of the next noise tile (32 rows x 64 keys fp32), one 16-byte slot per lane and
+  // load instruction: a lane reads back exactly the slots it filled
+  constexpr int kErWaveBytes = 32 * BN * 4;
+  __shared__ __align__(16) char ldsEr[kErLds ? WAVES * kErWaveBytes : 16];
 
   const int BH = p.B * p.H;
   const int nMB = (p.Sq + BM - 1) / BM;
@@ -134,6 +140,47 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     a_i = noise_row(nk, (uint32_t)qi);
   }
   if (KF == kKfTensor) er_row = p.exp_rand + b * p.er_sb + h * p.er_sh + (int64_t)qi_c * p.er_sr;
+  // kKfTensorLds: the wave's slice of a noise tile is 32 rows x 256 bytes.  Load r8 of a tile brings rows
+  // 4 r8 + [0..3] whole (a load instruction then touches 8 cache lines; with a lane fetching its own row's chunks
+  // it touched 32, and the address path, not HBM, bounded the pass): lane l fills slot l % 16 of row 4 r8 + l / 16
+  // with global chunk (l % 16) ^ (row % 16), the XOR placement that lets 32 rows be read back one chunk column at
+  // a time without bank conflicts.  Chunks past the end of a row re-read its last chunk (those keys are masked),
+  // rows past Sq the last row.
+  rsrc_t er_rsrc = make_rsrc(kErLds ? p.exp_rand + b * p.er_sb + h * p.er_sh : nullptr);
+  char* er_lds = ldsEr + (kErLds ? wave * kErWaveBytes : 0);
+  // per-lane state of those loads: two registers (the offsets of the eight loads are rebuilt from them for every
+  // tile: kept in registers across the loop they would cost eight, and this path has none to spare)
+  const int er_cs = (lane & 15) ^ (lane >> 4);  // slot ^ (row % 4); the row's bits 2..3 are those of r8
+  const uint32_t er_row_bytes = (uint32_t)p.er_sr * 4u;
+  const uint32_t er_off0 = kErLds ? (uint32_t)(m0 + wave * 32 + (lane >> 4)) * er_row_bytes : 0u;
+  const uint32_t er_off_last = kErLds ? (uint32_t)(p.Sq - 1) * er_row_bytes : 0u;
+  auto issue_er = [&](int t) __attribute__((always_inline)) {
+    const int last_chunk = p.Skv / 4 - 1;
+    int cs = er_cs;
+    uint32_t off0 = er_off0;
+    asm volatile("" : "+v"(cs), "+v"(off0));  // not loop-invariant as far as the compiler can tell
+#pragma unroll
+    for (int r8 = 0; r8 < 8; ++r8) {
+      const int c = min(t * (BN / 4) + (cs ^ (4 * (r8 & 3))), last_chunk);
+      const uint32_t row_off = min(off0 + (uint32_t)(4 * r8) * er_row_bytes, er_off_last);
+      load_lds16(er_rsrc, er_lds + r8 * 1024, row_off + (uint32_t)c * 16u, 0);
+    }
+  };
+  // the lane's query row n, chunks 2 k8 + g (keys 8 k8 + 4 g + [0..3] of the tile: score registers 4 (k8 % 4) + [0..3]
+  // of half k8 / 4)
+  // (slot (2 k8 + g) ^ (n % 16) of row n: byte offset ((g ^ n % 16) << 4) ^ (k8 << 5) inside the row, so one
+  // register and one xor with a constant per read)
+  const uint32_t er_rd0 = (uint32_t)(n * 256) | (uint32_t)((g ^ (n & 15)) << 4);
+  auto read_er = [&](float (&dst)[2][16]) __attribute__((always_inline)) {
+    uint32_t rd0 = er_rd0;
+    asm volatile("" : "+v"(rd0));
+#pragma unroll
+    for (int k8 = 0; k8 < 8; ++k8) {
+      const float4v e4 = *reinterpret_cast<const float4v*>(er_lds + (rd0 ^ (uint32_t)(k8 << 5)));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[k8 >> 2][4 * (k8 & 3) + e] = e4[e];
+    }
+  };
 
   TileStager<D, BN, NT, kRowSwizzle> stK;
   TileStager<D, BN, NT, kTrSwizzle> stV;
@@ -422,7 +469,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         float log2E;
-        if (KF == kKfTensor) {
+        if (kTensor) {
           log2E = __builtin_amdgcn_logf(er[r]);
         } else {
           const int jl = 32 * mbk + 8 * (r >> 2) + 4 * g + (r & 3);
@@ -648,6 +695,14 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     constexpr bool odd = decltype(odd_tag)::value;
     wait_vmem();
     __syncthreads();
+    if (kErLds && it < nw) {
+      // this tile's slice from LDS to registers, then the next tile's on its way into the same slots: in flight
+      // for the whole tile without holding a register.  The reads must have returned before the loads may
+      // overwrite their slots (nothing in the hardware orders an LDS read against a later direct-to-LDS load).
+      read_er(er);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      if (it + 1 < nw) issue_er(it + 1);
+    }
     stage_k(it + 1, odd ? ldsK0 : ldsK1);
     stage_v(it + 1, odd ? ldsV0 : ldsV1);
     if (it < nw) {  // not entirely above this wave's diagonal
@@ -669,6 +724,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
     load_er_half(er[0], 0, 0);
     load_er_half(er[1], 0, 1);
   }
+  if (kErLds && nw > 0) issue_er(0);
   stage_k(0, ldsK0);
   stage_v(0, ldsV0);
   int it = 0;
@@ -699,7 +755,7 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES) attn_fwd_kernel(const A
       }
     if (g == 0 && p.lse) p.lse[(int64_t)bh * p.Sq + qi] = m_run + __builtin_amdgcn_logf(l_run);
   }
-  if (KF == kKfTensor || kSeeded) {
+  if (kTensor || kSeeded) {
     l_kf += xchg32(l_kf);
     if (KF == kKfSeededTau1) l_kf *= -kLog2e;  // the sum was taken over 1 / log2 u = -ln2 / E
     // packed modes: the perturbed sum shares the plain softmax's stabiliser, scaled by 1 / tau
@@ -725,12 +781,14 @@ hipError_t launch_one(const AttnKernelParams& p0, hipStream_t stream) {
   const int64_t BH = (int64_t)p.B * p.H;
   // 256-row workgroups (8 waves) halve the K/V staging per row (measured 148 vs 158 us at B1 H32 S4096), but
   // there are half as many of them: used on the pipelined paths once they still fill the chip twice
-  constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast;
+  // (kKfTensorLds: the noise slices in flight through LDS leave room for one workgroup per CU in either form, so the
+  // 256-row one is used as soon as there is a workgroup for every CU)
+  constexpr bool kHas8 = KF == kKfNone || KF == kKfSoftcap || KF == kKfSeededTau1 || KF == kKfSeededFast || KF == kKfTensorLds;
   if constexpr (kHas8) {
     const int nMB8 = (p.Sq + 255) / 256;
     const int64_t n8 = (int64_t)nMB8 * BH;
     const int64_t cus = device_cu_count();
-    if ((forced & 7) ? (forced & 7) >= 2 : n8 >= 2 * cus) {
+    if ((forced & 7) ? (forced & 7) >= 2 : n8 >= (KF == kKfTensorLds ? cus : 2 * cus)) {
       // causal: pair the heaviest block with the lightest inside one workgroup when the pairs come out as whole
       // rounds of the chip (or as many rounds that a ragged last one does not matter)
       const int64_t pairs = (int64_t)((nMB8 + 1) / 2) * BH;
@@ -757,6 +815,7 @@ hipError_t launch_td(const AttnKernelParams& p, bool causal, bool emu, int kf, h
   if (causal == C && emu == E && kf == K) return launch_one<T, D, C, E, K>(p, s);
   FT_CASE(true, true, kKfNone) FT_CASE(true, false, kKfNone) FT_CASE(false, true, kKfNone) FT_CASE(false, false, kKfNone)
   FT_CASE(true, true, kKfTensor) FT_CASE(true, false, kKfTensor) FT_CASE(false, true, kKfTensor) FT_CASE(false, false, kKfTensor)
+  FT_CASE(true, true, kKfTensorLds) FT_CASE(true, false, kKfTensorLds) FT_CASE(false, true, kKfTensorLds) FT_CASE(false, false, kKfTensorLds)
   FT_CASE(true, true, kKfSeeded) FT_CASE(true, false, kKfSeeded) FT_CASE(false, true, kKfSeeded) FT_CASE(false, false, kKfSeeded)
   FT_CASE(true, true, kKfSoftcap) FT_CASE(true, false, kKfSoftcap) FT_CASE(false, true, kKfSoftcap) FT_CASE(false, false, kKfSoftcap)
   if constexpr (std::is_same<T, F16>::value) {  // packed KeyFormer modes: fp16 with reference rounding only

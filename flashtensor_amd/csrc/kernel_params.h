@@ -59,7 +59,9 @@ struct ColstatsKernelParams {
 // weight exp((t + g) / tau) with g = -ln E equals exp(t / tau) E^(-1/tau); the in-kernel E lies in
 // [6e-8, 16.7], so for tau >= 0.25 the plain softmax's running maximum also stabilises the perturbed sum
 // (exponent <= (6 + 24) / tau <= 120) and no second maximum is tracked; tau == 1 needs 1 / E only.
-enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2, kKfSoftcap = 3, kKfSeededTau1 = 4, kKfSeededFast = 5 };
+// kKfTensorLds: the noise tensor of kKfTensor, its tiles landing in LDS by direct-to-LDS loads a whole tile ahead
+// (16-byte aligned rows, Skv a multiple of 4, a (b, h) slice below 2 GiB; kKfTensor reads any layout into registers)
+enum KfMode { kKfNone = 0, kKfTensor = 1, kKfSeeded = 2, kKfSoftcap = 3, kKfSeededTau1 = 4, kKfSeededFast = 5, kKfTensorLds = 6 };
 // kStatCormRule: thresholds 1 / (i + 1) per query row i; kStatCormTensor: thresholds read from a tensor
 enum StatMode {
   kStatSum = 0, kStatSumSq = 1, kStatKfTensor = 2, kStatKfSeeded = 3, kStatCormRule = 4, kStatCormTensor = 5,

@@ -69,7 +69,9 @@ typedef struct FtAttnArgs {
  * positive and finite, pairs hidden by the causal mask included: the reference adds -log(exp_rand) to the whole
  * score matrix (kf.py:36-38), and the kernels may read any element of the tensor for a pair they then mask.
  * exp_rand == NULL: drawn in-kernel from the counter-based stream keyed by `seed`
- * (ft_noise_exp_fill* materialise the same tensor). */
+ * (ft_noise_exp_fill* materialise the same tensor).  That stream is this library's own definition (the reference
+ * has none: it takes the tensor as an input); it is fixed for a given FT_ABI_VERSION, and a change of the
+ * stream changes that version. */
 typedef struct FtNoise {
   const float* exp_rand;
   int64_t stride_b, stride_h, stride_row;

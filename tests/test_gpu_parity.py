@@ -88,6 +88,33 @@ def test_keyformer_small(gpu, B, S, H, D, seed, tau):
   assert torch.allclose(ed, es, rtol=2e-6, atol=0)
 
 
+@pytest.mark.parametrize("B,S,Skv,H,D,seed", [(1, 200, 200, 2, 128, 80), (2, 300, 364, 2, 64, 81), (1, 1100, 1100, 3, 128, 82),
+                                              (1, 520, 522, 2, 128, 83)])
+def test_keyformer_noise_tensor_layouts(gpu, monkeypatch, B, S, Skv, H, D, seed):
+  """The reference's own signature, forward(q, k, v, exp_rand).  Rows that can be fetched in 16-byte chunks reach
+  the attention pass through LDS a tile ahead (ragged last tile: chunks past the row end; Skv > Sq); a row stride
+  larger than Skv keeps that path; a view that starts 4 bytes off, or Skv not a multiple of 4, takes the register
+  path.  Every layout must give the same bits, in the 128-row and the 256-row form, and agree with the oracle."""
+  (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=seed, kv_len=Skv)
+  er = oracle.prepare_exp_rand(B, H, S, Skv, seed=seed)
+  ref_o, ref_s = oracle.keyformer_forward(q, k, v, er, tau=1.5)
+  erd = er.to(gpu)
+  wide = torch.zeros(B, H, S, Skv + 24, dtype=torch.float32, device=gpu)
+  wide[..., :Skv] = erd
+  off = torch.zeros(B * H * S * Skv + 1, dtype=torch.float32, device=gpu)
+  off[1:] = erd.flatten()
+  layouts = {"contiguous": erd, "wide rows": wide[..., :Skv], "offset by one float": off[1:].view(B, H, S, Skv)}
+  base = None
+  for form in ("4", "8"):
+    monkeypatch.setenv("FT_ATTN_FORM", form)
+    for name, e in layouts.items():
+      out, sc = ops.keyformer(qd, kd, vd, e, tau=1.5)
+      if base is None:
+        base = (out, sc)
+        check_o(out, ref_o); check_score(sc, ref_s)
+      assert torch.equal(out, base[0]) and torch.equal(sc, base[1]), (form, name)
+
+
 @pytest.mark.parametrize("tau", [0.2, 0.25, 0.5, 1.0, 4.0])
 def test_keyformer_seeded_paths(gpu, tau):
   """tau == 1 and tau >= 0.25 take the packed path (no second running maximum), smaller tau the generic one;
@@ -770,18 +797,16 @@ def _take_pairs(t, pairs, head_axis):
 
 
 def test_headline_h2o_b1_h32_s4096_d128_with_topk(gpu):
-  """The benchmarked workload itself (H2O fp16, B1 H32 S4096 D128) against the oracle on 8 heads spread over
-  the XCDs, top-k k = S/8 by the gap rule, row-sum invariant on all heads."""
+  """The benchmarked workload itself (H2O fp16, B1 H32 S4096 D128) against the oracle on all 32 heads, top-k
+  k = S/8 by the gap rule, row-sum invariant."""
   S, H = 4096, 32
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, S, H, 128, seed=0)
   out, s = ops.h2o(qd, kd, vd)
   idx = ops.topk(s, S // 8)
-  pairs = [(0, h) for h in SPREAD_HEADS]
-  sub = tuple(_take_pairs(t, pairs, 2) for t in (q, k, v))
-  ref_o, ref_s = oracle.chunked_over_heads(oracle.h2o_forward, sub, head_chunk=4)
-  check_o(_take_pairs(out.cpu(), pairs, 2), ref_o)
-  check_score(_take_pairs(s.cpu(), pairs, 1), ref_s)
-  assert oracle.topk_agreement(_take_pairs(idx.cpu(), pairs, 1), ref_s, S // 8) == 0
+  ref_o, ref_s = oracle.chunked_over_heads(oracle.h2o_forward, (q, k, v), head_chunk=4)
+  check_o(out, ref_o)
+  check_score(s, ref_s)
+  assert oracle.topk_agreement(idx.cpu(), ref_s, S // 8) == 0
   assert torch.allclose(s.sum(-1).cpu(), torch.full((1, H), float(S)), rtol=1e-4)
   assert torch.equal(out[:, 0].cpu(), v[:, 0])
 
@@ -807,24 +832,26 @@ def test_config3_keyformer_b1_h32_s4096_d128_tau1(gpu):
   # (the two paths differ in how the row sums are accumulated: fp32 exps vs the fp16 P fed to the MFMA)
   assert torch.allclose(s_ones, s_h2o, rtol=2e-4, atol=1e-7)
   del ones
-  # tensor noise, reference recipe and default tau, oracle on the first and last heads
-  HS = 2
-  tp = [(0, 0), (0, 31)]
-  er = oracle.prepare_exp_rand(1, HS, S, S, seed=1)
+  # tensor noise, reference recipe and default tau, oracle on four heads of different XCD residues
+  tp = [(0, 0), (0, 13), (0, 22), (0, 31)]
+  er = oracle.prepare_exp_rand(1, len(tp), S, S, seed=1)
   big = torch.ones(1, H, S, S, dtype=torch.float32, device=gpu)
-  big[:, 0] = er[:, 0].to(gpu)
-  big[:, 31] = er[:, 1].to(gpu)
-  _, s_t = ops.keyformer(qd, kd, vd, big, tau=1.5)
-  _, ref_t = oracle.keyformer_forward(*(_take_pairs(t, tp, 2) for t in (q, k, v)), er, tau=1.5)
-  check_score(_take_pairs(s_t.cpu(), tp, 1), ref_t)
+  for n, (_, h) in enumerate(tp):
+    big[:, h] = er[:, n].to(gpu)
+  out_t, s_t = ops.keyformer(qd, kd, vd, big, tau=1.5)
+  for i in range(0, len(tp), 2):
+    pp = tp[i:i + 2]
+    ref_to, ref_t = oracle.keyformer_forward(*(_take_pairs(t, pp, 2) for t in (q, k, v)), er[:, i:i + 2], tau=1.5)
+    check_o(_take_pairs(out_t.cpu(), pp, 2), ref_to); check_score(_take_pairs(s_t.cpu(), pp, 1), ref_t)
 
 
 def test_config4_roco_b4_h32_s4096_d128(gpu):
   B, S, H = 4, 4096, 32
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, 128, seed=0)
   out, s1, s2 = ops.roco(qd, kd, vd)
-  # 8 (b, h) pairs: batches 0 and 3 plus one each of 1 and 2, heads on different XCD residues
-  pairs = [(0, 0), (0, 7), (0, 31), (1, 8), (2, 15), (3, 0), (3, 24), (3, 31)]
+  # 16 (b, h) pairs: four of every batch, heads on different XCD residues
+  pairs = [(0, 0), (0, 7), (0, 18), (0, 31), (1, 3), (1, 8), (1, 21), (1, 30), (2, 1), (2, 15), (2, 20), (2, 26),
+           (3, 0), (3, 13), (3, 24), (3, 31)]
   sub = tuple(_take_pairs(t, pairs, 2) for t in (q, k, v))
   ref_o, r1, r2 = oracle.chunked_over_heads(oracle.roco_forward, sub, head_chunk=4)
   check_o(_take_pairs(out.cpu(), pairs, 2), ref_o)
