@@ -1,6 +1,6 @@
 """Benchmark of the fused attention + per-key score path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--calibrate-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs] [--no-split] [--calibrate-copy]
 
 A step is one H2O call (attention forward + column-statistics pass, the two launches behind
 ft_attn_colstats_fwd) on B=1, H=32, S=4096, D=128 fp16 inputs already resident in HBM.  Prints ONE JSON
@@ -88,7 +88,7 @@ def host_us_per_call(dev, calls=2000):
   return dt / calls * 1e6
 
 
-def per_config_table(dev, only=None, iters=100):
+def per_config_table(dev, only=None, iters=100, splits=True):
   """µs per call, algorithmic TFLOP/s and GB/s with their roofline fractions for the five configurations
   (`only`: just the rows whose name contains that text)."""
   import torch
@@ -109,7 +109,7 @@ def per_config_table(dev, only=None, iters=100):
     tf, gb = flops / us / 1e6, nbytes / us / 1e3
     rows.append({"config": name, "shape": shape, "us": round(us, 1), "tflops": round(tf, 1),
                  "mfma_frac": round(tf / PEAK_MFMA_TFLOPS, 4), "gbs": round(gb, 1), "hbm_frac": round(gb / PEAK_HBM_GBS, 4)})
-    if split:
+    if split and splits:
       rows[-1]["kernels_us"] = kernel_split(fn)
 
   def softmax_case(name, B, S, H, D, fn_of, extra_bytes=0, split=False):
@@ -250,6 +250,9 @@ def main():
   ap.add_argument("--cpu-heads", type=int, default=4)
   ap.add_argument("--only", default=None, help="per-configuration table: only the rows whose name contains this text")
   ap.add_argument("--config-iters", type=int, default=100, help="timed calls per row of the per-configuration table")
+  ap.add_argument("--no-split", action="store_true",
+                  help="per-configuration table without the per-kernel split (which attaches torch's profiler: leave it "
+                       "out when the whole run is already under rocprofv3)")
   ap.add_argument("--calibrate-copy", action="store_true",
                   help="also run a 256 MiB device-to-device tensor copy a few times: under rocprofv3 --pmc its "
                        "FETCH_SIZE / WRITE_SIZE readings give the counter unit for the other kernels")
@@ -347,7 +350,7 @@ def main():
   except Exception as e:  # diagnostic only: never costs the line
     result["mfma_probe"] = {"error": f"{type(e).__name__}: {e}"}
   if not args.no_configs:
-    result["per_config"] = per_config_table(dev, args.only, args.config_iters)
+    result["per_config"] = per_config_table(dev, args.only, args.config_iters, not args.no_split)
   result["cpu_baseline"] = cpu
   print(json.dumps(result))
 

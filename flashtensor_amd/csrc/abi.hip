@@ -485,15 +485,21 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
     return fail(FT_EUNSUPPORTED, "head_dim %d not supported by the linear-attention kernels (64, or 32 in adjacent pairs)", a->D);
   if (a->D == 32 && ((a->H & 1) || a->sq.h != 32 || a->sk.h != 32 || a->sv.h != 32 || a->so.h != 32))
     return fail(FT_EUNSUPPORTED, "head_dim 32 needs an even number of heads stored 32 elements apart (H=%d)", a->H);
-  if (a->dtype != FT_F16) return fail(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16)", a->dtype);
-  if (out_dtype != FT_F16 && out_dtype != FT_F32) return fail(FT_EUNSUPPORTED, "out_dtype must be f16 or f32");
+  if (a->dtype != FT_F16 && a->dtype != FT_BF16 && a->dtype != FT_F32)
+    return fail(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16, bf16 or f32)", a->dtype);
+  if (out_dtype != a->dtype && out_dtype != FT_F32)
+    return fail(FT_EUNSUPPORTED, "out_dtype must be the input type or f32 (got %d for inputs of type %d)", out_dtype, a->dtype);
   if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->o))
     return fail(FT_EINVAL, "q, k, v, o must be 16-byte aligned");
-  if (!stride_ok(a->sq) || !stride_ok(a->sk) || !stride_ok(a->sv) || !stride_ok(a->so))
-    return fail(FT_EINVAL, "strides must be positive multiples of 8 elements with a contiguous head_dim axis");
-  if ((int64_t)a->Sq * a->sq.s * 2 >= 0x7fffffffLL || (int64_t)a->Sq * a->sk.s * 2 >= 0x7fffffffLL ||
-      (int64_t)a->Sq * a->sv.s * 2 >= 0x7fffffffLL)
-    return fail(FT_EUNSUPPORTED, "sequence stride too large: S * stride_s must stay below 2^30 elements");
+  // rows are moved in 16-byte pieces: strides in multiples of 8 elements for 16-bit tensors, of 4 for fp32 ones
+  const int64_t in_mul = a->dtype == FT_F32 ? 4 : 8, out_mul = out_dtype == FT_F32 ? 4 : 8;
+  auto strides_ok = [](const FtStrides& s, int64_t m) { return s.b % m == 0 && s.s % m == 0 && s.h % m == 0 && s.s > 0; };
+  if (!strides_ok(a->sq, in_mul) || !strides_ok(a->sk, in_mul) || !strides_ok(a->sv, in_mul) || !strides_ok(a->so, out_mul))
+    return fail(FT_EINVAL, "strides must be positive multiples of 16 bytes with a contiguous head_dim axis");
+  const int64_t esz = a->dtype == FT_F32 ? 4 : 2;
+  if ((int64_t)a->Sq * a->sq.s * esz >= 0x7fffffffLL || (int64_t)a->Sq * a->sk.s * esz >= 0x7fffffffLL ||
+      (int64_t)a->Sq * a->sv.s * esz >= 0x7fffffffLL)
+    return fail(FT_EUNSUPPORTED, "sequence stride too large: S * stride_s must stay below 2^31 bytes");
   const size_t need = ft::linattn_workspace_bytes(*a, kind);
   if (!workspace || workspace_bytes < need)
     return fail(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);

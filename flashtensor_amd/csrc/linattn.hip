@@ -1,5 +1,7 @@
-// Linear-attention cores EA and SimA for gfx950, fp16, head_dim 64 (head_dim 32 as pairs of adjacent heads:
-// the merge step drops the two cross-head blocks of the 64x64 matrix, the output step keeps EA's softmax per half).
+// Linear-attention cores EA and SimA for gfx950, head_dim 64 (head_dim 32 as pairs of adjacent heads: the merge
+// step drops the two cross-head blocks of the 64x64 matrix, the output step keeps EA's softmax per half).
+// fp16 or bf16 tensors (the harness's type switch, cases/attn.py:90,97) with MFMA operands of the same type, or
+// fp32 tensors (the type of bench/ea.mlir:2, bench/sima.mlir:2), rounded to fp16 as they are loaded.
 //
 // Replaces the fused kernels the reference would emit for bench/ea.mlir:13-17 and bench/sima.mlir:13-17
 // (asuka.softmax / asuka.normalize semantics: lib/Dialect/Asuka/Transforms/LowerComplexReduce.cpp:21-69):
@@ -115,10 +117,14 @@ __device__ __forceinline__ void wave_lds_order() {
 // One wave's private strip of ROWS tokens x 64 channels (128-byte rows): lane l moves the 16-byte chunk
 // l % 8 of rows l / 8 + 8 i, global -> registers -> LDS, so every load instruction covers 8 whole rows.
 // Rows past the end of the sequence re-read the last token (callers mask them).
-template <int ROWS, int SWZ>
+// IN32: the tensor holds fp32 (256-byte rows); a lane then loads the 32 bytes behind its chunk and rounds them to
+// eight fp16 values when the strip is parked in LDS, so that everything downstream sees the 16-bit layout.
+template <int ROWS, int SWZ, bool IN32 = false>
 struct StripMover {
   typedef TileGeom<kLinD> G;
   static constexpr int ROUNDS = ROWS / 8;
+  static constexpr int LOADS = IN32 ? 2 * ROUNDS : ROUNDS;  // 16-byte loads per lane and strip
+  typedef uint4v Regs[LOADS];
   const char* base;
   int64_t row_bytes;
   int last_row;
@@ -128,11 +134,11 @@ struct StripMover {
 
   __device__ __forceinline__ void init(const uint16_t* base_, int64_t row_stride, int rows_total) {
     base = reinterpret_cast<const char*>(base_);
-    row_bytes = row_stride * 2;
+    row_bytes = row_stride * (IN32 ? 4 : 2);
     last_row = rows_total - 1;
     const int lane = lane_id();
     r_lane = lane >> 3;
-    c16 = (lane & 7) * 16;
+    c16 = (lane & 7) * (IN32 ? 32 : 16);
 #pragma unroll
     for (int it = 0; it < ROUNDS; ++it) {
       const int r = it * 8 + r_lane;
@@ -145,25 +151,59 @@ struct StripMover {
   // prefetch unconditionally (a fixed number of loads in flight, which the compiler can count: with loads that
   // may or may not have been issued it waits for all of them) without touching another wave's rows
   __device__ __forceinline__ void limit_rows(int last) { last_row = max(0, min(last_row, last)); }
-  __device__ __forceinline__ void load(int row0, uint4v (&regs)[ROUNDS]) const {
+  __device__ __forceinline__ void load(int row0, Regs& regs) const {
 #pragma unroll
     for (int it = 0; it < ROUNDS; ++it) {
       const int r = min(row0 + it * 8 + r_lane, last_row);
-      regs[it] = *reinterpret_cast<const uint4v*>(base + r * row_bytes + c16);
+      if (IN32) {
+        regs[2 * it] = *reinterpret_cast<const uint4v*>(base + r * row_bytes + c16);
+        regs[2 * it + 1] = *reinterpret_cast<const uint4v*>(base + r * row_bytes + c16 + 16);
+      } else {
+        regs[it] = *reinterpret_cast<const uint4v*>(base + r * row_bytes + c16);
+      }
     }
   }
-  __device__ __forceinline__ void to_lds(const uint4v (&regs)[ROUNDS], char* lds_strip) const {
+  // the lane's eight 16-bit elements of round `it`
+  __device__ __forceinline__ uint4v chunk16(const Regs& regs, int it) const {
+    if (!IN32) return regs[it];
+    // (whole vectors are reinterpreted, then indexed: a bit cast applied to one element of a vector lvalue read
+    // element 0 whatever the index)
+    const float4v lo = __builtin_bit_cast(float4v, regs[2 * it]), hi = __builtin_bit_cast(float4v, regs[2 * it + 1]);
+    const uint4v out = {F16::pack2(lo[0], lo[1]), F16::pack2(lo[2], lo[3]), F16::pack2(hi[0], hi[1]), F16::pack2(hi[2], hi[3])};
+    return out;
+  }
+  __device__ __forceinline__ void to_lds(const Regs& regs, char* lds_strip) const {
 #pragma unroll
-    for (int it = 0; it < ROUNDS; ++it) *reinterpret_cast<uint4v*>(lds_strip + lds_off[it]) = regs[it];
+    for (int it = 0; it < ROUNDS; ++it) *reinterpret_cast<uint4v*>(lds_strip + lds_off[it]) = chunk16(regs, it);
   }
 };
 
+// fp16-only packed maximum of the 8 elements of an operand, or the same through fp32 for bf16
+template <typename T>
+__device__ __forceinline__ float max8(typename T::vec8 v) {
+  if constexpr (__is_same(typename T::elem, _Float16)) {
+    half2v hm = __builtin_elementwise_max(__builtin_shufflevector(v, v, 0, 1), __builtin_shufflevector(v, v, 2, 3));
+    hm = __builtin_elementwise_max(hm, __builtin_shufflevector(v, v, 4, 5));
+    hm = __builtin_elementwise_max(hm, __builtin_shufflevector(v, v, 6, 7));
+    return fmaxf((float)hm[0], (float)hm[1]);
+  } else {
+    float m = (float)v[0];
+#pragma unroll
+    for (int s = 1; s < 8; ++s) m = fmaxf(m, (float)v[s]);
+    return m;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // NQ: also accumulate sum_s |Q| (SimA with normalised queries).
-template <bool EA, bool NQ>
+// T: element type of the MFMA operands (F16 or BF16); IN32: the tensors hold fp32 and are rounded to fp16 on the way.
+template <typename T, bool IN32, bool EA, bool NQ>
 __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinParams p) {
+  static_assert(!IN32 || __is_same(typename T::elem, _Float16), "fp32 tensors are rounded to fp16 operands");
+  typedef typename T::vec8 vec8;
   constexpr int D = kLinD, STEP = 16;
-  constexpr int P = NQ ? 2 : 3;               // strips in flight per wave (three tensors at three strips each do not fit in registers)
+  // strips in flight per wave (three tensors at three strips each do not fit in registers, nor do fp32 strips)
+  constexpr int P = (NQ || IN32) ? 2 : 3;
   constexpr int STRIP = STEP * 2 * D;         // 2 KB
   constexpr int R = STEP / 8;                 // 16-byte loads per lane, strip and tensor
   __shared__ __align__(16) char s_kv[kLinWaves][2 * STRIP];  // wave-private K and V strips
@@ -199,13 +239,15 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 #pragma unroll
   for (int e = 0; e < 8; ++e) qabs[e] = 0.f;
 
-  StripMover<STEP, kTrSwizzle> mvK, mvV;
-  StripMover<STEP, kNoSwizzle> mvQ;
-  mvK.init(p.k + b * p.sk.b + h * p.sk.h, p.sk.s, p.S);
-  mvV.init(p.v + b * p.sv.b + h * p.sv.h, p.sv.s, p.S);
-  if (NQ) mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
+  StripMover<STEP, kTrSwizzle, IN32> mvK, mvV;
+  StripMover<STEP, kNoSwizzle, IN32> mvQ;
+  constexpr int RL = IN32 ? 2 * R : R;  // 16-byte loads per lane, strip and tensor
+  constexpr int ES = IN32 ? 2 : 1;  // tensor element size in units of the 16-bit pointer type
+  mvK.init(p.k + (b * p.sk.b + h * p.sk.h) * ES, p.sk.s, p.S);
+  mvV.init(p.v + (b * p.sv.b + h * p.sv.h) * ES, p.sv.s, p.S);
+  if (NQ) mvQ.init(p.q + (b * p.sq.b + h * p.sq.h) * ES, p.sq.s, p.S);
 
-  uint4v rk[P][R], rv[P][R], rq[P][R];  // strips in flight, indexed by compile-time slot
+  uint4v rk[P][RL], rv[P][RL], rq[P][RL];  // strips in flight, indexed by compile-time slot
   auto strip_row0 = [&](int i) { return tok_begin + (wave + kLinWaves * i) * STEP; };
   {
     const int last_mine = nmine > 0 ? strip_row0(nmine - 1) + STEP - 1 : tok_begin;
@@ -224,12 +266,12 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
   // one strip, already in the wave's LDS buffer: TAIL = some of its tokens lie past the end
   auto compute = [&](auto tail_tag, int t0) {
     constexpr bool TAIL = decltype(tail_tag)::value;
-    half8 ka[2];
+    vec8 ka[2];
 #pragma unroll
-    for (int db = 0; db < 2; ++db) ka[db] = read_tr_operand<D, half8>(tk, 0, 32 * db);
-    half8 vb[2];
+    for (int db = 0; db < 2; ++db) ka[db] = read_tr_operand<D, vec8>(tk, 0, 32 * db);
+    vec8 vb[2];
 #pragma unroll
-    for (int eb = 0; eb < 2; ++eb) vb[eb] = read_tr_operand<D, half8>(tv, 0, 32 * eb);
+    for (int eb = 0; eb < 2; ++eb) vb[eb] = read_tr_operand<D, vec8>(tv, 0, 32 * eb);
     bool dead[8];  // token slot s of this lane is past the end
 #pragma unroll
     for (int s = 0; s < 8; ++s) dead[s] = TAIL && t0 + 4 * g + (s & 3) + ((s >> 2) << 3) >= p.S;
@@ -244,10 +286,7 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 #pragma unroll
           for (int s = 0; s < 8; ++s) mx = fmaxf(mx, dead[s] ? NEG_INF : (float)ka[db][s]);
         } else {
-          half2v hm = __builtin_elementwise_max(__builtin_shufflevector(ka[db], ka[db], 0, 1), __builtin_shufflevector(ka[db], ka[db], 2, 3));
-          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(ka[db], ka[db], 4, 5));
-          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(ka[db], ka[db], 6, 7));
-          mx = fmaxf((float)hm[0], (float)hm[1]);
+          mx = max8<T>(ka[db]);
         }
         mx = fmaxf(mx, xchg32(mx));
         m_new[db] = fmaxf(m_run[db], mx);
@@ -283,7 +322,6 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
           }
         wave_lds_order();
       }
-      const half2v ones = {(_Float16)1.f, (_Float16)1.f};
 #pragma unroll
       for (int db = 0; db < 2; ++db) {
         const float mb = m_run[db] * kLog2e;
@@ -294,26 +332,24 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
           float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf((float)ka[db][2 * j + 1], kLog2e, -mb));
           if (dead[2 * j]) e0 = 0.f;
           if (dead[2 * j + 1]) e1 = 0.f;
-          const float2v e2 = {e0, e1};
-          const half2v ph = __builtin_convertvector(e2, half2v);
-          l_run[db] = __builtin_amdgcn_fdot2(ph, ones, l_run[db], false);  // sum of the fp16 values the MFMA consumes
-          pw[j] = __builtin_bit_cast(uint32_t, ph);
+          pw[j] = T::pack2(e0, e1);
+          l_run[db] = T::add2(pw[j], l_run[db]);  // sum of the 16-bit values the MFMA consumes
         }
-        ka[db] = __builtin_bit_cast(half8, pw);
+        ka[db] = __builtin_bit_cast(vec8, pw);
       }
     } else {
 #pragma unroll
       for (int db = 0; db < 2; ++db)
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-          if (dead[s]) ka[db][s] = (_Float16)0.f;
+          if (dead[s]) ka[db][s] = (typename T::elem)0.f;
           l_run[db] += __builtin_fabsf((float)ka[db][s]);
         }
     }
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
-      for (int eb = 0; eb < 2; ++eb) acc[db][eb] = F16::mfma(ka[db], vb[eb], acc[db][eb]);
+      for (int eb = 0; eb < 2; ++eb) acc[db][eb] = T::mfma(ka[db], vb[eb], acc[db][eb]);
   };
 
   // strip i has been fetched into register slot SLOT: park it in LDS, refill the slot with strip i + P (past
@@ -329,7 +365,7 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
       // a lane holds channels 8 (lane % 8) + [0..7] of rows lane / 8 (+ 8) of the strip
 #pragma unroll
       for (int it = 0; it < R; ++it) {
-        const half8 qv = __builtin_bit_cast(half8, rq[SLOT][it]);
+        const vec8 qv = __builtin_bit_cast(vec8, mvQ.chunk16(rq[SLOT], it));
         const bool live = i < nmine && (!tail || t0 + it * 8 + (lane >> 3) < p.S);  // not a re-read row past the share
 #pragma unroll
         for (int e = 0; e < 8; ++e) qabs[e] += live ? __builtin_fabsf((float)qv[e]) : 0.f;
@@ -480,7 +516,11 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinPar
 
 // ---------------------------------------------------------------------------------------------------
 // One workgroup per (b, h, block of 16 output channels).
-template <bool EA>
+// T: type of the W operand pair written for the output pass: hi = T(x), lo = T((x - hi) 2^kLoShift), i.e. 22
+// significant bits as fp16 + fp16 and 16 as bf16 + bf16
+template <typename T> constexpr int kLoShift = __is_same(typename T::elem, _Float16) ? 11 : 8;
+
+template <typename T, bool EA>
 __global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinParams p, int normalize_q) {
   constexpr int D = kLinD, EB = 16, TS = D + 8;
   __shared__ float s_scale[D];   // per-channel factor applied to the summed matrix
@@ -591,10 +631,10 @@ __global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinPar
   for (int i = 0; i < 4; ++i) {
     const int idx = t + i * kLinThreads;
     const float x = accv[i] * scale;
-    const _Float16 hi = (_Float16)x;
-    const _Float16 lo = (_Float16)((x - (float)hi) * 2048.f);
-    s_t[0][idx % EB][drow[i]] = __builtin_bit_cast(uint16_t, hi);
-    s_t[1][idx % EB][drow[i]] = __builtin_bit_cast(uint16_t, lo);
+    const uint16_t hi = T::from_float(x);
+    const uint16_t lo = T::from_float((x - T::to_float(hi)) * (float)(1 << kLoShift<T>));
+    s_t[0][idx % EB][drow[i]] = hi;
+    s_t[1][idx % EB][drow[i]] = lo;
   }
   __syncthreads();
   {
@@ -605,8 +645,10 @@ __global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinPar
 }
 
 // ---------------------------------------------------------------------------------------------------
-template <bool EA, bool F32OUT>
+template <typename T, bool IN32, bool EA, bool F32OUT>
 __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinParams p) {
+  static_assert(!IN32 || __is_same(typename T::elem, _Float16), "fp32 tensors are rounded to fp16 operands");
+  typedef typename T::vec8 vec8;
   constexpr int D = kLinD, SUB = 32;
   constexpr int P = 2;                           // Q strips in flight per wave
   constexpr int STRIP = SUB * 2 * D;             // 4 KB
@@ -653,18 +695,19 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   for (int i = 0; i < 4; ++i) winv[i] = p.winv[bh * 4 + i];
   // A operand: W^T[e][d], hi and lo, rows e = 32 eb + n, contraction slots d = 16 t + 8 g + [0..7]
   const uint16_t* w = p.w + (int64_t)bh * 2 * D * D;
-  half8 whi[2][4], wlo[2][4];
+  vec8 whi[2][4], wlo[2][4];
 #pragma unroll
   for (int eb = 0; eb < 2; ++eb)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      whi[eb][t] = *reinterpret_cast<const half8*>(w + (32 * eb + n) * D + 16 * t + 8 * g);
-      if (F32OUT) wlo[eb][t] = *reinterpret_cast<const half8*>(w + D * D + (32 * eb + n) * D + 16 * t + 8 * g);
+      whi[eb][t] = *reinterpret_cast<const vec8*>(w + (32 * eb + n) * D + 16 * t + 8 * g);
+      if (F32OUT) wlo[eb][t] = *reinterpret_cast<const vec8*>(w + D * D + (32 * eb + n) * D + 16 * t + 8 * g);
     }
 
-  StripMover<SUB, kRowSwizzle> mvQ;
-  mvQ.init(p.q + b * p.sq.b + h * p.sq.h, p.sq.s, p.S);
-  uint4v rq[P][R];  // strips in flight, indexed by compile-time slot
+  StripMover<SUB, kRowSwizzle, IN32> mvQ;
+  mvQ.init(p.q + (b * p.sq.b + h * p.sq.h) * (IN32 ? 2 : 1), p.sq.s, p.S);
+  constexpr int RL = IN32 ? 2 * R : R;
+  uint4v rq[P][RL];  // strips in flight, indexed by compile-time slot
   auto strip_row0 = [&](int i) { return tok_begin + (strip0 + strip_step * i) * SUB; };
   mvQ.limit_rows(nmine > 0 ? strip_row0(nmine - 1) + SUB - 1 : tok_begin);
   __builtin_amdgcn_sched_barrier(0);  // scales and W, then strip 0, then strip 1: loads complete in the order they are issued
@@ -675,7 +718,10 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
   // the compiler, the wait for W sits inside the loop, in front of the MFMAs, where on every later trip it
   // waits for the strip requested a few instructions earlier instead.
   static_assert(P * R == 8, "the wait below counts the loads of the two strips");
-  __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8), every other counter at its maximum
+  if (IN32)
+    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): fp32 strips take twice the loads
+  else
+    __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8), every other counter at its maximum
 
   char* obase = static_cast<char*>(p.o) + (b * p.so.b + h * p.so.h) * (int64_t)(F32OUT ? 4 : 2);
   const int64_t orow_bytes = p.so.s * (int64_t)(F32OUT ? 4 : 2);
@@ -692,9 +738,9 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
     if (i >= nmine) return;  // past the wave's share: the slot has been moved and refilled, nothing to compute
 
     // B operand: f(Q)^T, column = token n, same contraction slots
-    half8 qf[4];
+    vec8 qf[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) qf[t] = read_row_chunk<D, half8>(tq, n, 2 * t + g);
+    for (int t = 0; t < 4; ++t) qf[t] = read_row_chunk<D, vec8>(tq, n, 2 * t + g);
 
     // EA: softmax over the 64 channels of the token.  The operand is the fp16 value of exp(q - max); the
     // division by the row sum (taken over those rounded values) is applied to the fp32 result.
@@ -704,34 +750,21 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
     if (EA) {
       float mx[2], sum[2] = {0.f, 0.f};
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        half2v hm = __builtin_shufflevector(qf[2 * hf], qf[2 * hf], 0, 1);
-#pragma unroll
-        for (int t = 2 * hf; t < 2 * hf + 2; ++t) {
-          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 0, 1));
-          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 2, 3));
-          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 4, 5));
-          hm = __builtin_elementwise_max(hm, __builtin_shufflevector(qf[t], qf[t], 6, 7));
-        }
-        mx[hf] = fmaxf((float)hm[0], (float)hm[1]);
-      }
+      for (int hf = 0; hf < 2; ++hf) mx[hf] = fmaxf(max8<T>(qf[2 * hf]), max8<T>(qf[2 * hf + 1]));
       if (!p.half_heads) mx[0] = mx[1] = fmaxf(mx[0], mx[1]);
       mx[0] = fmaxf(mx[0], xchg32(mx[0]));
       mx[1] = fmaxf(mx[1], xchg32(mx[1]));
-      const half2v ones = {(_Float16)1.f, (_Float16)1.f};
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const float mb = mx[t >> 1] * kLog2e;
         uint4v pw;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float2v e2 = {__builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j], kLog2e, -mb)),
-                              __builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j + 1], kLog2e, -mb))};
-          const half2v ph = __builtin_convertvector(e2, half2v);
-          sum[t >> 1] = __builtin_amdgcn_fdot2(ph, ones, sum[t >> 1], false);
-          pw[j] = __builtin_bit_cast(uint32_t, ph);
+          pw[j] = T::pack2(__builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j], kLog2e, -mb)),
+                           __builtin_amdgcn_exp2f(__builtin_fmaf((float)qf[t][2 * j + 1], kLog2e, -mb)));
+          sum[t >> 1] = T::add2(pw[j], sum[t >> 1]);
         }
-        qf[t] = __builtin_bit_cast(half8, pw);
+        qf[t] = __builtin_bit_cast(vec8, pw);
       }
       if (!p.half_heads) sum[0] = sum[1] = sum[0] + sum[1];
       sum[0] += xchg32(sum[0]);
@@ -753,8 +786,8 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int eb = 0; eb < 2; ++eb) {
-        ahi[eb] = F16::mfma(whi[eb][t], qf[t], ahi[eb]);
-        if (F32OUT) alo[eb] = F16::mfma(wlo[eb][t], qf[t], alo[eb]);
+        ahi[eb] = T::mfma(whi[eb][t], qf[t], ahi[eb]);
+        if (F32OUT) alo[eb] = T::mfma(wlo[eb][t], qf[t], alo[eb]);
       }
     float osc[4];
 #pragma unroll
@@ -769,14 +802,14 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
         float y[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          y[e] = (F32OUT ? ahi[eb][4 * q4 + e] + alo[eb][4 * q4 + e] * (1.f / 2048.f) : ahi[eb][4 * q4 + e]) * osc[2 * eb + (q4 >> 1)];
+          y[e] = (F32OUT ? ahi[eb][4 * q4 + e] + alo[eb][4 * q4 + e] * (1.f / (float)(1 << kLoShift<T>)) : ahi[eb][4 * q4 + e]) * osc[2 * eb + (q4 >> 1)];
         if (F32OUT) {
           float4v o4 = {y[0], y[1], y[2], y[3]};
           *reinterpret_cast<float4v*>(ost + n * OROW + e0 * 4) = o4;
         } else {
           uint2 pk;
-          pk.x = (uint32_t)F16::from_float(y[0]) | ((uint32_t)F16::from_float(y[1]) << 16);
-          pk.y = (uint32_t)F16::from_float(y[2]) | ((uint32_t)F16::from_float(y[3]) << 16);
+          pk.x = T::pack2(y[0], y[1]);
+          pk.y = T::pack2(y[2], y[3]);
           *reinterpret_cast<uint2*>(ost + n * OROW + e0 * 2) = pk;
         }
       }
@@ -801,6 +834,11 @@ __global__ void __launch_bounds__(kLinThreads, 2) linattn_out_kernel(const LinPa
     step(i + 1, std::integral_constant<int, 1>{});
   }
 }
+
+template <typename T>
+struct TypeTag {
+  typedef T type;
+};
 
 // ---------------------------------------------------------------------------------------------------
 hipError_t launch_linattn(const FtAttnArgs& a0, int kind, int normalize_q, int out_dtype, void* ws, hipStream_t s) {
@@ -840,33 +878,51 @@ hipError_t launch_linattn(const FtAttnArgs& a0, int kind, int normalize_q, int o
   p.winv = reinterpret_cast<float*>(base);
 
   const dim3 grid1((unsigned)(bh * p.nch)), grid3((unsigned)((p.out_wave_heads ? bh / kLinWaves : bh) * p.out_nch)), blk(kLinThreads);
-  if (ea)
-    hipLaunchKernelGGL((linattn_kv_kernel<true, false>), grid1, blk, 0, s, p);
-  else if (nq)
-    hipLaunchKernelGGL((linattn_kv_kernel<false, true>), grid1, blk, 0, s, p);
-  else
-    hipLaunchKernelGGL((linattn_kv_kernel<false, false>), grid1, blk, 0, s, p);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
   const dim3 grid2((unsigned)(bh * 4));
-  if (ea)
-    hipLaunchKernelGGL(linattn_merge_kernel<true>, grid2, blk, 0, s, p, 0);
+  hipError_t e = hipErrorInvalidValue;
+  // T: operand type; IN32: fp32 tensors (fp32 output only)
+  auto run = [&](auto t_tag, auto in32_tag) {
+    typedef typename decltype(t_tag)::type T;
+    constexpr bool IN32 = decltype(in32_tag)::value;
+    if (ea)
+      hipLaunchKernelGGL((linattn_kv_kernel<T, IN32, true, false>), grid1, blk, 0, s, p);
+    else if (nq)
+      hipLaunchKernelGGL((linattn_kv_kernel<T, IN32, false, true>), grid1, blk, 0, s, p);
+    else
+      hipLaunchKernelGGL((linattn_kv_kernel<T, IN32, false, false>), grid1, blk, 0, s, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return;
+    if (ea)
+      hipLaunchKernelGGL((linattn_merge_kernel<T, true>), grid2, blk, 0, s, p, 0);
+    else
+      hipLaunchKernelGGL((linattn_merge_kernel<T, false>), grid2, blk, 0, s, p, nq ? 1 : 0);
+    e = hipGetLastError();
+    if (e != hipSuccess) return;
+    if constexpr (IN32) {
+      if (ea)
+        hipLaunchKernelGGL((linattn_out_kernel<T, true, true, true>), grid3, blk, 0, s, p);
+      else
+        hipLaunchKernelGGL((linattn_out_kernel<T, true, false, true>), grid3, blk, 0, s, p);
+    } else if (ea) {
+      if (f32)
+        hipLaunchKernelGGL((linattn_out_kernel<T, false, true, true>), grid3, blk, 0, s, p);
+      else
+        hipLaunchKernelGGL((linattn_out_kernel<T, false, true, false>), grid3, blk, 0, s, p);
+    } else {
+      if (f32)
+        hipLaunchKernelGGL((linattn_out_kernel<T, false, false, true>), grid3, blk, 0, s, p);
+      else
+        hipLaunchKernelGGL((linattn_out_kernel<T, false, false, false>), grid3, blk, 0, s, p);
+    }
+    e = hipGetLastError();
+  };
+  if (a.dtype == FT_F32)
+    run(TypeTag<F16>{}, std::true_type{});
+  else if (a.dtype == FT_BF16)
+    run(TypeTag<BF16>{}, std::false_type{});
   else
-    hipLaunchKernelGGL(linattn_merge_kernel<false>, grid2, blk, 0, s, p, nq ? 1 : 0);
-  e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  if (ea) {
-    if (f32)
-      hipLaunchKernelGGL((linattn_out_kernel<true, true>), grid3, blk, 0, s, p);
-    else
-      hipLaunchKernelGGL((linattn_out_kernel<true, false>), grid3, blk, 0, s, p);
-  } else {
-    if (f32)
-      hipLaunchKernelGGL((linattn_out_kernel<false, true>), grid3, blk, 0, s, p);
-    else
-      hipLaunchKernelGGL((linattn_out_kernel<false, false>), grid3, blk, 0, s, p);
-  }
-  return hipGetLastError();
+    run(TypeTag<F16>{}, std::false_type{});
+  return e;
 }
 
 }  // namespace ft

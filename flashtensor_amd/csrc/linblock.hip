@@ -72,7 +72,7 @@ LtApi& lt_api() {
   return api;
 }
 
-// One Linear: y[M,N] = x[M,K] w[N,K]^T + bias[N], all row-major 16-bit, fp32 accumulation.  In the
+// One Linear: y[M,N] = x[M,K] w[N,K]^T + bias[N], all row-major and of one type (fp16, bf16 or fp32), fp32 accumulation.  In the
 // column-major terms of the library: D[N,M] = op_T(A = w as [K,N]) * (B = x as [K,M]), bias along D's rows.
 struct LinearPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
@@ -84,7 +84,7 @@ struct LinearPlan {
 struct LtState {
   std::mutex mu;
   std::map<int, hipblasLtHandle_t> handles;                               // per device
-  std::map<std::tuple<int, int64_t, int64_t, int64_t, bool>, LinearPlan> plans;  // (device, M, N, K, bias)
+  std::map<std::tuple<int, int64_t, int64_t, int64_t, bool, int>, LinearPlan> plans;  // (device, M, N, K, bias, dtype)
 };
 
 LtState& lt_state() {
@@ -99,8 +99,9 @@ LtState& lt_state() {
   } while (0)
 
 // Callers hold LtState::mu.
-int linear(LtApi& api, LtState& st, int device, const void* x, const void* w, const void* bias, void* y, int64_t M,
+int linear(LtApi& api, LtState& st, int device, int dtype, const void* x, const void* w, const void* bias, void* y, int64_t M,
            int64_t N, int64_t K, void* lt_ws, hipStream_t stream) {
+  const hipDataType lt_type = dtype == FT_F32 ? HIP_R_32F : dtype == FT_BF16 ? HIP_R_16BF : HIP_R_16F;
   hipblasLtHandle_t handle;
   auto hit = st.handles.find(device);
   if (hit == st.handles.end()) {
@@ -109,7 +110,7 @@ int linear(LtApi& api, LtState& st, int device, const void* x, const void* w, co
   } else {
     handle = hit->second;
   }
-  const auto key = std::make_tuple(device, M, N, K, bias != nullptr);
+  const auto key = std::make_tuple(device, M, N, K, bias != nullptr, dtype);
   auto pit = st.plans.find(key);
   if (pit == st.plans.end()) {
     LinearPlan p;
@@ -119,15 +120,15 @@ int linear(LtApi& api, LtState& st, int device, const void* x, const void* w, co
     LT_TRY(api.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n)), "transB");
     if (bias) {
       const uint32_t epi = HIPBLASLT_EPILOGUE_BIAS;
-      const int32_t bias_type = HIP_R_16F;
+      const int32_t bias_type = lt_type;
       LT_TRY(api.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi)), "epilogue");
       LT_TRY(api.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)), "bias type");
       // the heuristic wants a bias pointer in place; the real one is set before every call
       LT_TRY(api.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)), "bias pointer");
     }
-    LT_TRY(api.layout_create(&p.a, HIP_R_16F, (uint64_t)K, (uint64_t)N, K), "layout A");
-    LT_TRY(api.layout_create(&p.b, HIP_R_16F, (uint64_t)K, (uint64_t)M, K), "layout B");
-    LT_TRY(api.layout_create(&p.d, HIP_R_16F, (uint64_t)N, (uint64_t)M, N), "layout D");
+    LT_TRY(api.layout_create(&p.a, lt_type, (uint64_t)K, (uint64_t)N, K), "layout A");
+    LT_TRY(api.layout_create(&p.b, lt_type, (uint64_t)K, (uint64_t)M, K), "layout B");
+    LT_TRY(api.layout_create(&p.d, lt_type, (uint64_t)N, (uint64_t)M, N), "layout D");
     hipblasLtMatmulPreference_t pref;
     LT_TRY(api.pref_create(&pref), "preference creation");
     const uint64_t max_ws = kLtWorkspace;
@@ -137,8 +138,8 @@ int linear(LtApi& api, LtState& st, int device, const void* x, const void* w, co
     hipblasStatus_t hs = api.heuristic(handle, p.desc, p.a, p.b, p.d, p.d, pref, 1, res, &found);
     api.pref_destroy(pref);
     if (hs != HIPBLAS_STATUS_SUCCESS || found < 1)
-      return ft::set_error(FT_EUNSUPPORTED, "hipBLASLt has no kernel for a %lld x %lld x %lld f16 Linear (status %d)",
-                           (long long)M, (long long)N, (long long)K, (int)hs);
+      return ft::set_error(FT_EUNSUPPORTED, "hipBLASLt has no kernel for a %lld x %lld x %lld Linear of dtype %d (status %d)",
+                           (long long)M, (long long)N, (long long)K, dtype, (int)hs);
     p.algo = res[0].algo;
     p.workspace = res[0].workspaceSize;
     pit = st.plans.emplace(key, p).first;
@@ -157,7 +158,8 @@ int check_block(const FtLinBlockArgs* b, int kind) {
   if (b->B < 1 || b->S < 1 || b->H < 1) return ft::set_error(FT_EINVAL, "bad shape B=%d S=%d H=%d", b->B, b->S, b->H);
   if (b->D != 64 && !(b->D == 32 && (b->H & 1) == 0))
     return ft::set_error(FT_EUNSUPPORTED, "head_dim %d with %d heads not supported by the linear-attention kernels (64, or 32 with an even number of heads)", b->D, b->H);
-  if (b->dtype != FT_F16) return ft::set_error(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16)", b->dtype);
+  if (b->dtype != FT_F16 && b->dtype != FT_BF16 && b->dtype != FT_F32)
+    return ft::set_error(FT_EUNSUPPORTED, "dtype %d not supported by the linear-attention kernels (f16, bf16 or f32)", b->dtype);
   return FT_OK;
 }
 
@@ -170,13 +172,14 @@ BlockLayout block_layout(const FtLinBlockArgs& b, int kind, char* base) {
   BlockLayout l;
   const int64_t C = (int64_t)b.H * b.D;
   const size_t tokens = (size_t)b.B * b.S;
+  const size_t es = b.dtype == FT_F32 ? 4 : 2;
   l.qkv = 0;
-  l.core = l.qkv + align256(tokens * 3 * C * 2);
-  l.lin = l.core + align256(tokens * C * 2);
+  l.core = l.qkv + align256(tokens * 3 * C * es);
+  l.lin = l.core + align256(tokens * C * es);
   FtAttnArgs a{};
   a.q = base + l.qkv;
-  a.k = base + l.qkv + C * 2;
-  a.v = base + l.qkv + 2 * C * 2;
+  a.k = base + l.qkv + C * es;
+  a.v = base + l.qkv + 2 * C * es;
   a.o = base + l.core;
   a.sq = a.sk = a.sv = FtStrides{(int64_t)b.S * 3 * C, 3 * C, b.D};
   a.so = FtStrides{(int64_t)b.S * C, C, b.D};
@@ -221,11 +224,11 @@ int ft_linattn_block_fwd(const FtLinBlockArgs* b, int kind, int normalize_q, voi
   const int64_t C = (int64_t)b->H * b->D, M = (int64_t)b->B * b->S;
   LtState& st = lt_state();
   std::lock_guard<std::mutex> lock(st.mu);
-  rc = linear(api, st, device, b->x, b->w_qkv, b->b_qkv, base + l.qkv, M, 3 * C, C, base + l.lt, (hipStream_t)stream);
+  rc = linear(api, st, device, b->dtype, b->x, b->w_qkv, b->b_qkv, base + l.qkv, M, 3 * C, C, base + l.lt, (hipStream_t)stream);
   if (rc != FT_OK) return rc;
   rc = ft_linattn_fwd(&l.a, kind, normalize_q, b->dtype, base + l.lin, l.lt - l.lin, stream);
   if (rc != FT_OK) return rc;
-  return linear(api, st, device, base + l.core, b->w_out, b->b_out, b->y, M, C, C, base + l.lt, (hipStream_t)stream);
+  return linear(api, st, device, b->dtype, base + l.core, b->w_out, b->b_out, b->y, M, C, C, base + l.lt, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -13,6 +13,7 @@ import torch
 from . import _lib
 
 _DTYPES = {torch.float16: _lib.FT_F16, torch.bfloat16: _lib.FT_BF16}
+_LIN_DTYPES = {**_DTYPES, torch.float32: _lib.FT_F32}  # the linear cores also take the .mlir's own fp32
 
 
 def _k():
@@ -23,7 +24,7 @@ def _stream(t):
   return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def _check_qkv(q, k, v):
+def _check_qkv(q, k, v, dtypes=_DTYPES):
   for i, t in enumerate((q, k, v)):
     if not isinstance(t, torch.Tensor):
       raise RuntimeError(f"arg {i} need a torch.Tensor but got {type(t).__name__}")
@@ -33,8 +34,8 @@ def _check_qkv(q, k, v):
       raise RuntimeError(f"arg {i} need a GPU tensor but got device {t.device}")
     if t.dtype != q.dtype or t.device != q.device:
       raise RuntimeError(f"arg {i} need dtype {q.dtype} on {q.device} but got {t.dtype} on {t.device}")
-  if q.dtype not in _DTYPES:
-    raise RuntimeError(f"arg 0 need dtype float16 or bfloat16 but got {q.dtype}")
+  if q.dtype not in dtypes:
+    raise RuntimeError(f"arg 0 need dtype {' or '.join(str(d).split('.')[-1] for d in dtypes)} but got {q.dtype}")
   B, Sq, H, D = q.shape
   Hkv = k.shape[2]
   if tuple(k.shape) != (B, k.shape[1], Hkv, D) or Hkv < 1 or H % Hkv != 0:
@@ -54,15 +55,15 @@ def _dense_last(t):
 def _args(q, k, v, o, flags):
   B, Sq, H, D = q.shape
   return _k().AttnArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), q.stride()[:3], k.stride()[:3], v.stride()[:3],
-                       o.stride()[:3], B, H, Sq, k.shape[1], D, _DTYPES[q.dtype], flags, k.shape[2])
+                       o.stride()[:3], B, H, Sq, k.shape[1], D, _LIN_DTYPES[q.dtype], flags, k.shape[2])
 
 
 def _flags(causal, fast_logits):
   return (_lib.FT_CAUSAL if causal else 0) | (_lib.FT_FAST_LOGITS if fast_logits else 0)
 
 
-def _prep(q, k, v):
-  _check_qkv(q, k, v)
+def _prep(q, k, v, dtypes=_DTYPES):
+  _check_qkv(q, k, v, dtypes)
   return _dense_last(q), _dense_last(k), _dense_last(v)
 
 
@@ -173,21 +174,20 @@ def gemma2(q, k, v, softcap=50.0, causal=True, fast_logits=False):
 
 
 def _linattn(q, k, v, kind, normalize_q, out_dtype):
-  q, k, v = _prep(q, k, v)
+  q, k, v = _prep(q, k, v, _LIN_DTYPES)
   if q.shape[3] == 32:  # head_dim 32 runs as pairs of adjacent heads: heads must lie 32 elements apart
     for i, t in enumerate((q, k, v)):
       if t.stride(2) != 32:
         raise ValueError(f"arg {i} with head_dim 32 need heads stored 32 elements apart but got head stride {t.stride(2)}")
   ffi = _k()
   out_dtype = out_dtype or q.dtype
-  if out_dtype not in (torch.float16, torch.float32):
-    raise RuntimeError(f"out_dtype need float16 or float32 but got {out_dtype}")
+  if out_dtype not in (q.dtype, torch.float32):
+    raise RuntimeError(f"out_dtype need {q.dtype} or float32 but got {out_dtype}")
   out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
   a = _args(q, k, v, out, 0)
   nbytes = ffi.workspace_bytes(kind, a)
   ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-  ffi.linattn_fwd(a, kind, int(bool(normalize_q)), _lib.FT_F32 if out_dtype == torch.float32 else _lib.FT_F16, ws.data_ptr(),
-                  nbytes, _stream(q))
+  ffi.linattn_fwd(a, kind, int(bool(normalize_q)), _LIN_DTYPES[out_dtype], ws.data_ptr(), nbytes, _stream(q))
   return out
 
 
@@ -223,7 +223,9 @@ def _linattn_block(x, w_qkv, b_qkv, w_out, b_out, head_num, kind, normalize_q):
     if t is not None and not t.is_contiguous():
       raise ValueError(f"arg {i} ({name}) need a contiguous tensor but got strides {tuple(t.stride())}")
   y = torch.empty_like(x)
-  dt = {torch.float16: _lib.FT_F16, torch.bfloat16: _lib.FT_BF16}.get(x.dtype, _lib.FT_F32)
+  if x.dtype not in _LIN_DTYPES:
+    raise RuntimeError(f"arg 0 (x) need float16, bfloat16 or float32 but got {x.dtype}")
+  dt = _LIN_DTYPES[x.dtype]
   a = ffi.LinBlockArgs(x.data_ptr(), w_qkv.data_ptr(), 0 if b_qkv is None else b_qkv.data_ptr(), w_out.data_ptr(),
                        0 if b_out is None else b_out.data_ptr(), y.data_ptr(), B, S, head_num, C // head_num, dt)
   nbytes = ffi.linattn_block_workspace_bytes(a, kind)

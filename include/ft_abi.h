@@ -133,17 +133,20 @@ int ft_avgpool1d(const float* src, int64_t rows, int32_t S, int32_t kernel, floa
 
 /* Linear attention cores of bench/ea.mlir:13-17 (kind = FT_OP_EA) and bench/sima.mlir:13-17 (FT_OP_SIMA):
  * O = f(Q) (g(K)^T V).  normalize_q applies SimA's L1 normalisation to Q as well (ignored for EA).
- * out_dtype: FtDtype of o, FT_F16 or FT_F32.  fp16 inputs only (a->dtype == FT_F16); head_dim 64, or 32 (the
- * .mlir's own 4 heads of 32, :7-9) with an even number of heads stored 32 elements apart (s*.h == 32). */
+ * a->dtype: FT_F16 or FT_BF16 (the harness's type switch, cases/attn.py:90,97; MFMA operands of that type), or
+ * FT_F32, the type of the .mlir functions (ea.mlir:2): fp32 tensors are rounded to fp16 as they are loaded.
+ * out_dtype: FtDtype of o, the input type or FT_F32 (FT_F32 only for fp32 inputs).  Strides are multiples of 16
+ * bytes.  head_dim 64, or 32 (the .mlir's own 4 heads of 32, :7-9) with an even number of heads stored 32 elements
+ * apart (s*.h == 32). */
 int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype, void* workspace,
                    size_t workspace_bytes, void* stream);
 
 /* The whole block of bench/ea.mlir:2-23 / bench/sima.mlir:2-23 around the core: x [B,S,C] with C = H*D,
  * qkv = x w_qkv^T + b_qkv (w_qkv [3C,C] row-major as in a Linear, :3-5), split into q, k, v and into heads
- * (:6-12), the core (:13-17), y = core w_out^T + b_out (w_out [C,C], :20-22).  All tensors 16-bit and
- * contiguous; biases may be NULL.  The two projections are hipBLASLt GEMMs (fp32 accumulation, bias added
- * before the one rounding to 16 bits); q/k/v and the core's result live in the workspace as 16-bit tensors.
- * fp16; D = 64, or 32 with an even H. */
+ * (:6-12), the core (:13-17), y = core w_out^T + b_out (w_out [C,C], :20-22).  All tensors of one type (fp16,
+ * bf16, or the .mlir's own fp32) and contiguous; biases may be NULL.  The two projections are hipBLASLt GEMMs (fp32
+ * accumulation, bias added before the one rounding to the tensor type); q/k/v and the core's result live in the
+ * workspace as tensors of that type.  D = 64, or 32 with an even H. */
 typedef struct FtLinBlockArgs {
   const void* x;
   const void* w_qkv;

@@ -23,6 +23,8 @@ SHAPES = [("s128_d128", 1, 128, 2, 128, 0), ("s256_d64", 1, 256, 2, 64, 0), ("s2
 LIN_SHAPES = [("s256_d64", 1, 256, 2, 64, 0), ("s200_d64", 2, 200, 2, 64, 1)]
 NEXT_SHAPES = [("s128_d128", 1, 128, 2, 128, 3), ("s200_d64", 1, 200, 4, 64, 4)]
 BLOCK_SHAPES = [("s200_h2_d64", 2, 200, 2, 64, 5), ("s150_h4_d32", 1, 150, 4, 32, 6)]  # the second: head_dim 32, the .mlir's own
+# the linear cores and blocks in the other two types they take: bf16 (the harness's switch) and fp32 (the .mlir's own)
+DTYPE_SHAPES = [("s200_d64", 1, 200, 2, 64, 7)]
 KF_SEED = 1234
 
 
@@ -64,6 +66,17 @@ def main():
                         sima_block_rawq=oracle.sima_block_forward(*args, H, normalize_q=False).numpy(),
                         ea_core=oracle.ea_forward(q, k, v).numpy(),
                         sima_core=oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy())
+  for name, B, S, H, D, seed in DTYPE_SHAPES:
+    arrays = {}
+    for tag, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+      q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed, dtype=dt)
+      args = oracle.prepare_block_inputs(B, S, H, D, seed=seed, dtype=dt)
+      # numpy has no bf16: every result is stored as fp32 (a bf16 value is exactly representable)
+      arrays[f"ea_{tag}"] = oracle.ea_forward(q, k, v).float().numpy()
+      arrays[f"sima_{tag}_f32out"] = oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy()
+      arrays[f"ea_block_{tag}"] = oracle.ea_block_forward(*args, H).float().numpy()
+      arrays[f"sima_block_rawq_{tag}"] = oracle.sima_block_forward(*args, H, normalize_q=False).float().numpy()
+    np.savez_compressed(os.path.join(HERE, f"lindtype_{name}.npz"), B=B, S=S, H=H, D=D, seed=seed, **arrays)
   print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
 
 

@@ -132,6 +132,17 @@ def test_linattn_and_topk_argument_checks(lib):
   assert lib.ft_linattn_fwd(ctypes.byref(far), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EUNSUPPORTED
   c = _args(D=64, Sq=64, Skv=32, sq=st, sk=st, sv=st, so=st, flags=0)
   assert lib.ft_linattn_fwd(ctypes.byref(c), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, 1 << 20, None) == _lib.FT_EINVAL
+  # types: bf16 and fp32 tensors are taken; the output is of the input type or fp32; fp32 strides in multiples of 4
+  bf = _args(D=64, Sq=64, Skv=64, sq=st, sk=st, sv=st, so=st, flags=0, dtype=_lib.FT_BF16)
+  assert lib.ft_linattn_fwd(ctypes.byref(bf), _lib.FT_OP_EA, 1, _lib.FT_BF16, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
+  assert lib.ft_linattn_fwd(ctypes.byref(bf), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, need, None) == _lib.FT_EUNSUPPORTED
+  assert "out_dtype" in lib.ft_last_error().decode()
+  st4 = FtStrides(64 * 2 * 64 + 4, 2 * 64 + 4, 64)
+  f32 = _args(D=64, Sq=64, Skv=64, sq=st4, sk=st4, sv=st4, so=st4, flags=0, dtype=_lib.FT_F32)
+  assert lib.ft_linattn_fwd(ctypes.byref(f32), _lib.FT_OP_SIMA, 1, _lib.FT_F32, 0x5000, need - 1, None) == _lib.FT_EWORKSPACE
+  assert lib.ft_linattn_fwd(ctypes.byref(f32), _lib.FT_OP_SIMA, 1, _lib.FT_F16, 0x5000, need, None) == _lib.FT_EUNSUPPORTED
+  h4 = _args(D=64, Sq=64, Skv=64, sq=st4, sk=st4, sv=st4, so=st4, flags=0)   # 16-bit tensors need multiples of 8
+  assert lib.ft_linattn_fwd(ctypes.byref(h4), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, need, None) == _lib.FT_EINVAL
   assert lib.ft_topk(None, 1, 8, 2, 0x1000, None) == _lib.FT_EINVAL
   assert lib.ft_topk(0x1000, 1, 8, 9, 0x2000, None) == _lib.FT_EINVAL
   assert lib.ft_topk(0x1000, 1, 16384, 9, 0x2000, None) == _lib.FT_EUNSUPPORTED
@@ -156,6 +167,8 @@ def test_linear_block_argument_checks(lib):
   assert lib.ft_linattn_block_fwd(ctypes.byref(bad), _lib.FT_OP_SIMA, 1, 0x10000, need, None) == _lib.FT_EUNSUPPORTED
   odd = _lib.FtLinBlockArgs(0x1008, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
   assert lib.ft_linattn_block_fwd(ctypes.byref(odd), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
+  f32 = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F32)
+  assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(f32), _lib.FT_OP_EA) >= 2 * 100 * 4 * C * 4 + (32 << 20)
   nul = _lib.FtLinBlockArgs(0x1000, None, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
   assert lib.ft_linattn_block_fwd(ctypes.byref(nul), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
 

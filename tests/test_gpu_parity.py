@@ -403,6 +403,49 @@ def test_ea_sima_small(gpu, B, S, H, seed):
   assert torch.equal(ops.ea(qt, kt, vt), ops.ea(qd, kd, vd))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("B,S,H,D,seed", [(2, 200, 4, 64, 30), (1, 1000, 3, 64, 31), (1, 97, 2, 64, 32), (1, 300, 4, 32, 33),
+                                          (1, 2500, 2, 64, 34)])
+def test_ea_sima_bf16_and_fp32_tensors(gpu, dtype, B, S, H, D, seed):
+  """The other two types of the linear cores: bf16 (cases/attn.py:90,97; bf16 MFMA operands) and fp32, the type of
+  bench/ea.mlir:2 (rounded to fp16 operands on load: one fp16 rounding of every input, 2^-11 relative, which the
+  2e-3 bar on SimA's fp32 output allows for).  Outputs in the input type and in fp32."""
+  q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed, dtype=dtype)
+  qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+  o = ops.ea(qd, kd, vd)
+  assert o.dtype == dtype
+  check_o(o, oracle.ea_forward(q, k, v))
+  check_o(ops.ea(qd, kd, vd, out_dtype=torch.float32), oracle.ea_forward(q.float(), k.float(), v.float()))
+  rel = 2e-3 if dtype == torch.float32 else 1e-3
+  check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), oracle.sima_forward(q, k, v, out_dtype=torch.float32), rel=rel)
+  check_sima(ops.sima(qd, kd, vd, normalize_q=False, out_dtype=torch.float32),
+             oracle.sima_forward(q, k, v, normalize_q=False, out_dtype=torch.float32), rel=rel)
+  if dtype == torch.bfloat16:   # bf16 output: one bf16 step of the rounded fp32 reference
+    ref32 = oracle.sima_forward(q, k, v, out_dtype=torch.float32)
+    o16 = ops.sima(qd, kd, vd)
+    assert o16.dtype == torch.bfloat16
+    assert (o16.float().cpu() - ref32).abs().max().item() <= 8e-3 * ref32.abs().max().item()
+    with pytest.raises(RuntimeError):
+      ops.ea(qd, kd, vd, out_dtype=torch.float16)
+  if D == 64:  # a [B,H,S,D] storage order is a strided view of the same kernels: same bits
+    qt, kt, vt = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (qd, kd, vd))
+    assert torch.equal(ops.ea(qt, kt, vt), o)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "lindtype_*.npz"))), ids=os.path.basename)
+def test_linear_dtype_golden(gpu, path):
+  g = np.load(path, allow_pickle=False)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  for tag, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+    qd, kd, vd = (t.to(gpu) for t in oracle.prepare_inputs(B, S, H, D, seed=seed, dtype=dt))
+    check_o(ops.ea(qd, kd, vd), torch.from_numpy(g[f"ea_{tag}"]))
+    check_sima(ops.sima(qd, kd, vd, out_dtype=torch.float32), torch.from_numpy(g[f"sima_{tag}_f32out"]), rel=2e-3)
+    dev = tuple(t.to(gpu) for t in oracle.prepare_block_inputs(B, S, H, D, seed=seed, dtype=dt))
+    tight = 2e-2 if dt == torch.bfloat16 else 4e-3   # outputs of a few units: one bf16 step is 1.6e-2 there
+    check_o(ops.ea_block(*dev, H), torch.from_numpy(g[f"ea_block_{tag}"]), tight=tight)
+    check_o(ops.sima_block(*dev, H, normalize_q=False), torch.from_numpy(g[f"sima_block_rawq_{tag}"]), tight=tight)
+
+
 @pytest.mark.parametrize("B,S,H,seed", [(2, 200, 4, 20), (1, 333, 2, 21), (1, 784, 6, 22), (1, 1, 2, 23), (1, 300, 8, 24)])
 def test_ea_sima_head_dim_32(gpu, B, S, H, seed):
   """head_dim 32 (the literal shape of bench/ea.mlir:7-9) runs as pairs of adjacent heads on the 64-channel

@@ -76,5 +76,18 @@ def test_block_cases_match_golden(path):
   np.testing.assert_allclose(oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy(), g["sima_core"], rtol=1e-4, atol=1e-9)
 
 
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "lindtype_*.npz"))), ids=os.path.basename)
+def test_linear_cases_in_bf16_and_fp32_match_golden(path):
+  g = _load(path)
+  B, S, H, D, seed = (int(g[k]) for k in ("B", "S", "H", "D", "seed"))
+  for tag, dt, tol in (("bf16", torch.bfloat16, 8e-3), ("f32", torch.float32, 1e-5)):
+    q, k, v = oracle.prepare_inputs(B, S, H, D, seed=seed, dtype=dt)
+    args = oracle.prepare_block_inputs(B, S, H, D, seed=seed, dtype=dt)
+    assert np.abs(oracle.ea_forward(q, k, v).float().numpy() - g[f"ea_{tag}"]).max() <= tol
+    np.testing.assert_allclose(oracle.sima_forward(q, k, v, out_dtype=torch.float32).numpy(), g[f"sima_{tag}_f32out"], rtol=1e-4, atol=1e-9)
+    assert np.abs(oracle.ea_block_forward(*args, H).float().numpy() - g[f"ea_block_{tag}"]).max() <= 2 * tol
+    assert np.abs(oracle.sima_block_forward(*args, H, normalize_q=False).float().numpy() - g[f"sima_block_rawq_{tag}"]).max() <= 2 * tol
+
+
 def test_golden_files_present():
-  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 9
+  assert len(glob.glob(os.path.join(GOLDEN, "*.npz"))) == 10
