@@ -33,7 +33,7 @@ CASES_2D = {"attn_2d": kernels.Attn2D, "attn_h2o_2d": kernels.AttnH2O2D}
 
 def build(args, device):
   """Returns (callable, input tensors, algorithmic GFLOP, algorithmic GB) for the parsed options."""
-  dtype = torch.float16 if args.type == "f16" else torch.bfloat16
+  dtype = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[args.type]
   torch.manual_seed(0)
   esz = 2
   if args.model_name in CASES_2D:
@@ -80,7 +80,7 @@ def parse_args(argv=None):
   ap.add_argument("--kv_head_num", type=int, default=0)
   ap.add_argument("--head_dim", type=int, default=0)
   ap.add_argument("--masked", type=int, default=1)
-  ap.add_argument("--type", default="f16", choices=["f16", "bf16"])
+  ap.add_argument("--type", default="f16", choices=["f16", "bf16", "f32"], help="f32: the linear cases only (the type of bench/ea.mlir)")
   ap.add_argument("--run", type=int, default=10)
   ap.add_argument("--warmup", type=int, default=10)
   ap.add_argument("--show_result", action="store_true")
@@ -103,7 +103,7 @@ def load_check(args, device):
   args.batch_size, args.q_len, args.kv_len, args.head_num, args.head_dim = B, S, S, H, D
   g = torch.Generator(device="cpu")
   g.manual_seed(seed)
-  dtype = torch.float16 if args.type == "f16" else torch.bfloat16
+  dtype = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[args.type]
   inputs = [torch.randn(B, S, H, D, dtype=dtype, generator=g).to(device) for _ in range(3)]
   expected = []
   for key in CHECK_KEYS[args.model_name]:
