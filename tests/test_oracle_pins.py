@@ -307,6 +307,36 @@ def test_noise_stream_has_no_lattice_structure():
   assert stats.chisquare(np.bincount((low[:-1] * 16 + low[1:]).flatten(), minlength=256)).pvalue > 1e-4
 
 
+@pytest.mark.parametrize("seed", [1, 99, 2024, 123456789, 2 ** 40 + 7])
+def test_noise_stream_over_seeds_and_heads_and_its_multiplicative_relation(seed):
+  """The element word is a product a_i * b_j (mod 2^32) of a row and a column term, folded once.  Before the
+  fold the words of every 2x2 minor satisfy x_ij x_kl == x_il x_kj (mod 2^32) exactly; the emitted words and the
+  uniforms made of them must show nothing of it.  Checked for several seeds (one above 2^32) and (b, h) pairs."""
+  from scipy import stats
+  rng = np.random.default_rng(0)
+  for bh in (0, 5, 31):
+    x = oracle.noise_u32(seed, bh, np.arange(384), np.arange(384))
+    u = ((x >> np.uint32(9)).astype(np.float64) + 0.5) * 2.0 ** -23
+    assert stats.kstest(u.flatten()[::5], "uniform").pvalue > 1e-3
+    # products of the emitted words over 2x2 minors: never equal, top bytes agree at the chance rate 1/256
+    xa = (x[:-1, :-1].astype(np.uint64) * x[1:, 1:].astype(np.uint64)) & np.uint64(0xFFFFFFFF)
+    xb = (x[:-1, 1:].astype(np.uint64) * x[1:, :-1].astype(np.uint64)) & np.uint64(0xFFFFFFFF)
+    assert (xa == xb).mean() < 1e-4
+    agree = ((xa >> np.uint64(24)) == (xb >> np.uint64(24))).mean()
+    n = xa.size
+    assert abs(agree - 1 / 256) < 5 * math.sqrt((1 / 256) * (255 / 256) / n)
+    # the same relation in the domain the kernels use the numbers in: log u_ij + log u_kl - log u_il - log u_kj
+    # has the distribution it has for independent uniforms
+    L = np.log(u)
+    d = (L[:-1, :-1] + L[1:, 1:] - L[:-1, 1:] - L[1:, :-1]).flatten()[::7]
+    r = np.log(rng.random((4, d.size)))
+    assert stats.ks_2samp(d, r[0] + r[1] - r[2] - r[3]).pvalue > 1e-3
+    # different heads and different seeds do not share rows
+    other = oracle.noise_u32(seed, bh + 1, np.arange(384), np.arange(384))
+    assert (other == x).mean() < 1e-3
+  assert not np.array_equal(oracle.noise_u32(seed, 0, np.arange(8), np.arange(8)), oracle.noise_u32(seed + 1, 0, np.arange(8), np.arange(8)))
+
+
 # ------------------------------------------------------------------ SnapKV, CoRM, Gemma2
 
 def test_snapkv_pool_closed_forms_and_brute_force():
