@@ -125,8 +125,108 @@ __global__ void __launch_bounds__(NT) topk_kernel(const float* __restrict__ scor
   }
 }
 
+// Rows longer than the register sort holds (S > 8192), k <= kTopkSelectMax: one workgroup per row
+//   1. radix select over the 32-bit order keys, most significant byte first (four passes over the row, a 256-bin
+//      histogram in LDS each): the key T of the k-th entry and the number of entries that sort before it;
+//   2. one more pass gathers the winners into LDS as the 64-bit (order key, index) words of the register sort: every
+//      entry before T, and of the entries equal to T the ones with the smallest indices (a workgroup-wide prefix count
+//      in index order), as the full sort would have ranked them;
+//   3. a bitonic network over those <= 8192 words in LDS, and the indices go out in rank order.
+// The same answers as the register sort, ties and NaNs (which sort first, as in torch.topk) included.
+constexpr int kTopkSelectMax = 8192;
+constexpr int kTopkSelectThreads = 1024;
+
+__global__ void __launch_bounds__(kTopkSelectThreads) topk_select_kernel(const float* __restrict__ score, int S, int k,
+                                                                         int64_t* __restrict__ idx) {
+  constexpr int NT = kTopkSelectThreads, NW = NT / 64;
+  __shared__ uint64_t win[kTopkSelectMax];
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t wave_cnt[NW];
+  __shared__ uint32_t s_prefix, s_before, s_slot;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const float* row = score + (int64_t)blockIdx.x * S;
+
+  // ---- 1. the order key of rank k
+  uint32_t prefix = 0, before = 0;  // high bytes fixed so far; entries whose key is below every key with this prefix
+#pragma unroll 1
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (t < 256) hist[t] = 0;
+    __syncthreads();
+    const uint32_t mask = shift == 24 ? 0u : ~0u << (shift + 8);
+    for (int i = t; i < S; i += NT) {
+      const uint32_t h = float_order_desc(row[i]);
+      if ((h & mask) == prefix) atomicAdd(&hist[(h >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (t == 0) {
+      uint32_t cum = before, d = 0;
+      for (; d < 255; ++d) {
+        if (cum + hist[d] >= (uint32_t)k) break;
+        cum += hist[d];
+      }
+      s_prefix = prefix | (d << shift);
+      s_before = cum;
+    }
+    __syncthreads();
+    prefix = s_prefix;
+    before = s_before;
+  }
+  const uint32_t T = prefix;
+  const uint32_t need_eq = (uint32_t)k - before;  // entries equal to T that make the cut: those of smallest index
+
+  // ---- 2. gather
+  if (t == 0) s_slot = 0;
+  __syncthreads();
+  uint32_t eq_seen = 0;  // entries equal to T in the tiles before this one (the same in every thread)
+#pragma unroll 1
+  for (int i0 = 0; i0 < S; i0 += NT) {
+    const int i = i0 + t;
+    const uint32_t h = i < S ? float_order_desc(row[i]) : ~0u;
+    const bool lt = i < S && h < T, eq = i < S && h == T;
+    const uint64_t bal = __ballot(eq);
+    if (lane == 0) wave_cnt[wave] = (uint32_t)__popcll(bal);
+    __syncthreads();
+    uint32_t rank = eq_seen + (uint32_t)__popcll(bal & ((1ull << lane) - 1ull)), tile_eq = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      if (w < wave) rank += wave_cnt[w];
+      tile_eq += wave_cnt[w];
+    }
+    if (lt || (eq && rank < need_eq)) win[atomicAdd(&s_slot, 1u)] = ((uint64_t)h << 32) | (uint32_t)i;
+    eq_seen += tile_eq;
+    __syncthreads();
+  }
+  // ---- 3. sort the k winners (padding sorts last)
+  int n2 = 2;
+  while (n2 < k) n2 <<= 1;
+  for (int i = k + t; i < n2; i += NT) win[i] = ~0ull;
+  __syncthreads();
+#pragma unroll 1
+  for (int size = 2; size <= n2; size <<= 1)
+#pragma unroll 1
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int p = t; p < (n2 >> 1); p += NT) {
+        const int lo = ((p & ~(stride - 1)) << 1) | (p & (stride - 1)), hi = lo | stride;
+        const bool up = (lo & size) == 0;
+        const uint64_t a = win[lo], b = win[hi];
+        if ((a > b) == up) {
+          win[lo] = b;
+          win[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  int64_t* out = idx + (int64_t)blockIdx.x * k;
+  for (int i = t; i < k; i += NT) out[i] = (int64_t)(uint32_t)win[i];
+}
+
 hipError_t launch_topk(const float* score, int64_t rows, int S, int k, int64_t* idx, hipStream_t s) {
   const dim3 grid((unsigned)rows);
+  if (S > 8192) {
+    if (k > kTopkSelectMax) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(topk_select_kernel, grid, dim3(kTopkSelectThreads), 0, s, score, S, k, idx);
+    return hipGetLastError();
+  }
   if (S <= 512)
     hipLaunchKernelGGL((topk_kernel<2, 256>), grid, dim3(256), 0, s, score, S, k, idx);
   else if (S <= 1024)

@@ -198,7 +198,9 @@ __device__ __forceinline__ float max8(typename T::vec8 v) {
 // NQ: also accumulate sum_s |Q| (SimA with normalised queries).
 // T: element type of the MFMA operands (F16 or BF16); IN32: the tensors hold fp32 and are rounded to fp16 on the way.
 template <typename T, bool IN32, bool EA, bool NQ>
-__global__ void __launch_bounds__(kLinThreads, 2) linattn_kv_kernel(const LinParams p) {
+// (fp32 tensors with the |Q| sums keep three fp32 strips of two slots in flight: one workgroup per CU, so that the wave
+// has the accumulation registers as well and nothing spills)
+__global__ void __launch_bounds__(kLinThreads, (IN32 && NQ) ? 1 : 2) linattn_kv_kernel(const LinParams p) {
   static_assert(!IN32 || __is_same(typename T::elem, _Float16), "fp32 tensors are rounded to fp16 operands");
   typedef typename T::vec8 vec8;
   constexpr int D = kLinD, STEP = 16;
