@@ -226,6 +226,47 @@ def test_strided_views_and_bhsd_layout(gpu):
   check_o(out, ref_o); check_score(s1, r1)
 
 
+def test_operands_are_never_copied_behind_the_caller(gpu):
+  """A tensor the kernels cannot read in place is refused (ValueError, the C ABI's FT_EINVAL) by every operator:
+  a strided last axis of q / k / v, of the noise tensor and of CoRM's thresholds, non-contiguous operands of the
+  block operators, non-contiguous scores for top-k."""
+  B, S, H, D = 1, 64, 2, 64
+  (_, _, _), (qd, kd, vd) = gpu_inputs(gpu, B, S, H, D, seed=3)
+  wide = torch.randn(B, S, H, 2 * D, device=gpu).half()
+  bad = wide[..., ::2]                                   # last axis strided by two elements
+  assert bad.shape == qd.shape and bad.stride(-1) == 2
+  calls = {"attn": ops.attn, "h2o": ops.h2o, "roco": ops.roco, "keyformer": ops.keyformer, "snapkv": ops.snapkv,
+           "corm": ops.corm, "gemma2": ops.gemma2, "ea": ops.ea, "sima": ops.sima}
+  for name, f in calls.items():
+    for pos in range(3):
+      operands = [qd, kd, vd]
+      operands[pos] = bad
+      with pytest.raises(ValueError, match="contiguous last axis"):
+        f(*operands)
+  er = 1 + torch.randn(B, H, S, 2 * S, device=gpu).abs()
+  with pytest.raises(ValueError, match="contiguous last axis"):
+    ops.keyformer(qd, kd, vd, er[..., ::2])
+  thr = torch.rand(S, 2 * S, device=gpu)
+  with pytest.raises(ValueError, match="contiguous last axis"):
+    ops.corm(qd, kd, vd, thr[:, ::2])
+  C = H * D
+  x = torch.randn(2, S, C, device=gpu).half()
+  wq, bq = torch.randn(3 * C, C, device=gpu).half() / 8, torch.randn(3 * C, device=gpu).half()
+  wo, bo = torch.randn(C, C, device=gpu).half() / 8, torch.randn(C, device=gpu).half()
+  xt = x.transpose(0, 1).contiguous().transpose(0, 1)
+  assert not xt.is_contiguous()
+  for f in (ops.ea_block, ops.sima_block):
+    f(x, wq, bq, wo, bo, H)
+    for operands in ((xt, wq, bq, wo, bo), (x, wq.t().contiguous().t(), bq, wo, bo), (x, wq, bq, wo.t().contiguous().t(), bo),
+                     (x, wq, torch.randn(6 * C, device=gpu).half()[::2], wo, bo)):
+      with pytest.raises(ValueError, match="contiguous tensor"):
+        f(*operands, H)
+  with pytest.raises(ValueError, match="contiguous tensor"):
+    ops.topk(torch.randn(4, 128, device=gpu)[:, ::2], 8)
+  with pytest.raises(ValueError, match="contiguous tensor"):
+    ops.topk(torch.randn(64, 4, device=gpu).t(), 8)
+
+
 def test_bf16_inputs(gpu):
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 192, 2, 128, seed=9, dtype=torch.bfloat16)
   ref_o, r1 = oracle.h2o_forward(q, k, v)
@@ -770,6 +811,8 @@ def test_every_launch_form_of_the_attention_pass_on_ragged_shapes(gpu, monkeypat
     res[form] = (out, s1)
     if D == 128:
       res[form] += (ops.gemma2(qd, kd, vd),)
+      if form in ("4", "8"):  # the packed seeded KeyFormer modes (tau = 1 and tau != 1)
+        res[form] += ops.keyformer(qd, kd, vd, None, tau=1.0, seed=5) + ops.keyformer(qd, kd, vd, None, tau=1.5, seed=5)
   monkeypatch.delenv("FT_ATTN_FORM")
   auto = ops.h2o(qd, kd, vd)
   for form, r in res.items():
