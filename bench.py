@@ -161,14 +161,23 @@ def per_config_table(dev, only=None, iters=100, splits=True):
   add("5b ea block (projections + core)", "B8 S8192 C1024 H16", lambda: ops.ea_block(x, wq, bq, wo, bo, 16), blk_flops, blk_bytes)
   add("5b sima block", "B8 S8192 C1024 H16", lambda: ops.sima_block(x, wq, bq, wo, bo, 16, normalize_q=False), blk_flops, blk_bytes)
   del x, wq, wo, bq, bo
-  # the literal shape of bench/ea.mlir:2 (x [64,784,128], 4 heads of 32), in fp16
+  # the literal shape of bench/ea.mlir:2 (x [64,784,128], 4 heads of 32), in fp16: the two-launch form for narrow models
   C, M = 128, 64 * 784
   x = torch.randn(64, 784, C, dtype=torch.float16, device=dev)
   wq = (torch.randn(3 * C, C, device=dev) / C ** 0.5).half()
   wo = (torch.randn(C, C, device=dev) / C ** 0.5).half()
   bq, bo = torch.zeros(3 * C, dtype=torch.float16, device=dev), torch.zeros(C, dtype=torch.float16, device=dev)
+  c_flops = 2 * 2.0 * 64 * 4 * 784 * 32 * 32 + 2.0 * M * 4 * C * C
   add("5c ea block, .mlir shape", "B64 S784 C128 H4 D32", lambda: ops.ea_block(x, wq, bq, wo, bo, 4),
-      2 * 2.0 * 64 * 4 * 784 * 32 * 32 + 2.0 * M * 4 * C * C, (2.0 * M * C + 4 * C * C + 4 * C) * 2)
+      c_flops, (2.0 * M * C + 4 * C * C + 4 * C) * 2)
+  add("5c sima block, .mlir shape", "B64 S784 C128 H4 D32", lambda: ops.sima_block(x, wq, bq, wo, bo, 4),
+      c_flops, (2.0 * M * C + 4 * C * C + 4 * C) * 2)
+  # ... and in the .mlir's own type
+  xf, wqf, wof, bqf, bof = (t.float() for t in (x, wq, wo, bq, bo))
+  add("5c ea block, .mlir shape and type (f32)", "B64 S784 C128 H4 D32", lambda: ops.ea_block(xf, wqf, bqf, wof, bof, 4),
+      c_flops, (2.0 * M * C + 4 * C * C + 4 * C) * 4)
+  add("5c sima block, .mlir shape and type (f32)", "B64 S784 C128 H4 D32", lambda: ops.sima_block(xf, wqf, bqf, wof, bof, 4),
+      c_flops, (2.0 * M * C + 4 * C * C + 4 * C) * 4)
   return rows
 
 

@@ -16,7 +16,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libflashtensor_hip.so")
 DIAG_LIB_PATH = os.path.join(HERE, "libflashtensor_diag.so")  # include/ft_diag.h: probes for the benchmark, not product
 SOURCES = ["abi.hip", "attn_fwd.hip", "attn_fwd_f16_d128.hip", "attn_fwd_f16_d64.hip", "attn_fwd_bf16_d128.hip", "attn_fwd_bf16_d64.hip",
-           "colstats.hip", "linattn.hip", "aux.hip", "linblock.hip"]
+           "colstats.hip", "linattn.hip", "aux.hip", "linblock.hip", "linblock_small.hip"]
 DIAG_SOURCES = ["diag.hip"]
 FFI_SOURCE = "ffi_kernels.cpp"  # pybind11 module ft_ffi over the C ABI (plain C++: no device code, no torch headers)
 HEADERS = ["device_common.hpp", "kernel_params.h", "noise.h", "attn_fwd_kernel.hpp", os.path.join("..", "..", "include", "ft_abi.h"),

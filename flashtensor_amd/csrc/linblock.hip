@@ -4,6 +4,7 @@
 // with a bias epilogue and go to hipBLASLt; the library is opened with dlopen on first use so that the rest
 // of this library neither links against it nor needs it.
 #include <dlfcn.h>
+#include <stdlib.h>
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 
@@ -15,6 +16,10 @@
 
 namespace ft {
 int set_error(int code, const char* fmt, ...);
+// linblock_small.hip: the two-launch form for heads of 32 channels and C <= 128
+void small_block_plan(const FtLinBlockArgs& a, int* nch, int* strips_per_chunk);
+size_t small_block_workspace_bytes(const FtLinBlockArgs& a);
+hipError_t launch_small_block(const FtLinBlockArgs& a, int kind, int normalize_q, void* ws, hipStream_t s);
 }
 
 namespace {
@@ -214,6 +219,18 @@ int ft_linattn_block_fwd(const FtLinBlockArgs* b, int kind, int normalize_q, voi
   BlockLayout l = block_layout(*b, kind, static_cast<char*>(workspace));
   if (!workspace || workspace_bytes < l.total)
     return ft::set_error(FT_EWORKSPACE, "workspace of %zu bytes needed, got %zu", l.total, workspace ? workspace_bytes : (size_t)0);
+  {
+    // narrow models (the .mlir's own 4 heads of 32): weights in LDS, q / k / v in registers, two launches.
+    // FT_LINBLOCK_FORM=gemm in the environment is a test hook that keeps the library-GEMM form for them.
+    int nch = 0, spc = 0;
+    ft::small_block_plan(*b, &nch, &spc);
+    const char* form = getenv("FT_LINBLOCK_FORM");
+    if (nch > 0 && ft::small_block_workspace_bytes(*b) <= workspace_bytes && !(form && form[0] == 'g')) {
+      hipError_t le = ft::launch_small_block(*b, kind, normalize_q, workspace, (hipStream_t)stream);
+      if (le != hipSuccess) return ft::set_error(FT_ELAUNCH, "linear block launch: %s", hipGetErrorString(le));
+      return FT_OK;
+    }
+  }
   LtApi& api = lt_api();
   if (api.missing) return ft::set_error(FT_EUNSUPPORTED, "hipBLASLt is not available (%s not found)", api.missing);
   int device = 0;

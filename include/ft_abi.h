@@ -146,7 +146,11 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
  * (:6-12), the core (:13-17), y = core w_out^T + b_out (w_out [C,C], :20-22).  All tensors of one type (fp16,
  * bf16, or the .mlir's own fp32) and contiguous; biases may be NULL.  The two projections are hipBLASLt GEMMs (fp32
  * accumulation, bias added before the one rounding to the tensor type); q/k/v and the core's result live in the
- * workspace as tensors of that type.  D = 64, or 32 with an even H. */
+ * workspace as tensors of that type.  D = 64, or 32 with an even H.
+ * Narrow models (D = 32 with 2 or 4 heads, the .mlir's own geometry, and batches enough to fill the chip) run as
+ * two launches of this library's own instead: projection weights in LDS, q / k / v never leave registers, MFMA
+ * operands of the tensor type (fp16 for fp32 tensors: x and the weights are rounded as they are loaded), no
+ * hipBLASLt involved. */
 typedef struct FtLinBlockArgs {
   const void* x;
   const void* w_qkv;
@@ -161,8 +165,8 @@ typedef struct FtLinBlockArgs {
 /* 0 if the arguments are not supported (ft_last_error() says why). */
 size_t ft_linattn_block_workspace_bytes(const FtLinBlockArgs* b, int kind);
 
-/* hipBLASLt is opened on first use (FT_EUNSUPPORTED if it cannot be found); its handle and the GEMM plans
- * are cached per device and shape, and calls of this entry point serialise on one mutex. */
+/* Where the projections are library GEMMs, hipBLASLt is opened on first use (FT_EUNSUPPORTED if it cannot be found);
+ * its handle and the GEMM plans are cached per device and shape, and those calls serialise on one mutex. */
 int ft_linattn_block_fwd(const FtLinBlockArgs* b, int kind, int normalize_q, void* workspace, size_t workspace_bytes,
                          void* stream);
 

@@ -53,3 +53,9 @@ def test_linear_attention_kernels_do_not_spill():
   for name, r in res.items():
     if "linattn_" in name:
       assert r["vgpr_spill"] == 0 and r["scratch_bytes"] == 0, (name, r)
+  # the two-launch block for narrow models: 8 waves per workgroup, so two per SIMD must fit
+  res = _load("linblock_small.hip")
+  assert len([n for n in res if "linblk_" in n]) == 30
+  for name, r in res.items():
+    if "linblk_" in name:
+      assert r["vgpr_spill"] == 0 and r["scratch_bytes"] == 0 and r["occupancy"] >= 2, (name, r)

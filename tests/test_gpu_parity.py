@@ -536,6 +536,41 @@ def test_linear_block_mlir_literal_shape(gpu):
     check_o(ys[b:b + 1], oracle.sima_block_forward(*hb, H, normalize_q=False))
 
 
+@pytest.mark.parametrize("B,S,H,dtype,seed", [(64, 784, 4, torch.float32, 40), (64, 784, 4, torch.bfloat16, 41), (40, 100, 2, torch.float16, 42),
+                                              (70, 333, 4, torch.float16, 43), (300, 64, 2, torch.float32, 44), (130, 31, 4, torch.float16, 45),
+                                              (256, 1, 2, torch.float16, 46)])
+def test_linear_block_narrow_models_both_forms(gpu, monkeypatch, B, S, H, dtype, seed):
+  """Heads of 32 channels with C <= 128 and enough batches take the two-launch form (weights in LDS, q / k / v in
+  registers); FT_LINBLOCK_FORM=gemm keeps the library-GEMM form for the same call.  Both are checked against the
+  oracle on three batches: ragged strips, one token per batch, 2 and 4 heads, every tensor type, with and without
+  biases, both SimA readings.  (fp32 tensors: the two-launch form rounds x and the weights to fp16 MFMA operands,
+  the library form q, k, v: the same order of error, 2-6e-4 of the result's norm.)"""
+  host = oracle.prepare_block_inputs(B, S, H, 32, seed=seed, dtype=dtype)
+  dev = tuple(t.to(gpu) for t in host)
+  pick = (0, B // 2, B - 1)
+  tight = 2e-2 if dtype == torch.bfloat16 else 4e-3
+  calls = [("ea", lambda d: ops.ea_block(*d, H), lambda h: oracle.ea_block_forward(*h, H)),
+           ("sima raw q", lambda d: ops.sima_block(*d, H, normalize_q=False), lambda h: oracle.sima_block_forward(*h, H, normalize_q=False)),
+           ("sima", lambda d: ops.sima_block(*d, H), lambda h: oracle.sima_block_forward(*h, H))]
+  nobias = lambda t: (t[0], t[1], None, t[3], None)
+  for name, f, ref in calls:
+    for strip in (False, True):
+      d, h = (nobias(dev), nobias(host)) if strip else (dev, host)
+      if S == 1 and name != "ea":
+        continue  # one token: K / sum|K| is the sign of K, and a sign of a rounded near-zero is not a stable quantity
+      monkeypatch.delenv("FT_LINBLOCK_FORM", raising=False)
+      y = f(d)
+      monkeypatch.setenv("FT_LINBLOCK_FORM", "gemm")
+      yg = f(d)
+      monkeypatch.delenv("FT_LINBLOCK_FORM")
+      assert y.dtype == dtype and y.shape == (B, S, 32 * H) and torch.isfinite(y).all()
+      for b in pick:
+        want = ref((h[0][b:b + 1],) + tuple(h[1:]))
+        check_o(y[b:b + 1], want, tight=tight)
+        check_o(yg[b:b + 1], want, tight=tight)
+      assert rel_fro(y.float().cpu(), yg.float().cpu()) <= (6e-3 if dtype == torch.bfloat16 else 2e-3), name
+
+
 def test_ea_sima_properties(gpu):
   (q, k, v), (qd, kd, vd) = gpu_inputs(gpu, 1, 512, 2, 64, seed=5)
   c = torch.full_like(vd, 0.75)
