@@ -2,7 +2,8 @@
 // :20-22) in two launches for narrow models: C = H * 32 <= 128 channels, the geometry of the .mlir itself
 // (x [64,784,128], 4 heads of 32).  With so few channels the projection weights fit in LDS and a token's q, k, v never
 // leave the registers they are computed in, so x is read twice and y written once; nothing else touches HBM but a
-// few MB of per-chunk partial matrices.
+// few MB of per-chunk partial matrices.  x and y pass through a wave-private LDS tile on the way in and out, so that
+// every load and store instruction covers whole 128- or 256-byte row segments.
 //
 //   pass 1 (linblk_kv_kernel), one workgroup per (batch, token chunk), a wave per strip of 32 tokens:
 //     K = x Wk^T + bk and V = x Wv^T + bv with the tokens as MFMA rows, so that a lane ends up holding one channel
@@ -60,13 +61,64 @@ __device__ __forceinline__ uint4v load8(const void* base, int64_t elem) {
   }
 }
 
-// A lane's share of a 32-token strip of x as it lies in memory (token l % 32, channels 16 s + 8 g + [0..7] for every
-// step s), requested one strip ahead and turned into MFMA operands when the strip's turn comes.
-template <bool IN32, int KS>
+__device__ __forceinline__ void wave_lds_order() {  // for the compiler; a wave's LDS instructions execute in order
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// A 32-token strip of x on its way to a wave: requested one strip ahead with loads that cover whole rows (lane l takes
+// a 16-byte chunk of row l / CPR + RPI i: an instruction touches 8 cache lines; with every lane reading its own
+// token's row it touched 32, and the address path showed), parked in the wave's LDS tile when the strip's turn comes
+// (16-bit elements, the chunk placement of TileGeom's kRowSwizzle) and read back as MFMA operands: token l % 32,
+// channels 16 s + 8 g + [0..7] for step s.
+template <typename T, bool IN32, int C>
 struct XStrip {
-  static constexpr int N = IN32 ? 2 * KS : KS;
+  typedef TileGeom<C> G;
+  static constexpr int CPR = C * (IN32 ? 4 : 2) / 16;  // 16-byte chunks per row in memory
+  static constexpr int RPI = 64 / CPR;                 // rows per load instruction
+  static constexpr int N = kSbStrip / RPI;
+  static constexpr int kTileBytes = kSbStrip * G::RB;
   uint4v raw[N];
-  __device__ __forceinline__ void load(const void* x, int64_t elem0) {
+  // tok0: first token of the strip; rows past `last` (the batch's last token) re-read it
+  __device__ __forceinline__ void load(const void* x, int64_t batch_row0, int tok0, int last) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int64_t r = batch_row0 + min(tok0 + lane / CPR + RPI * i, last);
+      raw[i] = *reinterpret_cast<const uint4v*>(static_cast<const char*>(x) + (r * CPR + lane % CPR) * 16);
+    }
+  }
+  __device__ __forceinline__ void to_lds(char* tile) const {
+    const int lane = lane_id();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int r = lane / CPR + RPI * i, c = lane % CPR;
+      if constexpr (IN32) {  // 4 floats -> half a 16-byte chunk of 16-bit elements
+        const float4v v = __builtin_bit_cast(float4v, raw[i]);
+        *reinterpret_cast<uint2*>(tile + r * G::RB + (((c >> 1) ^ G::row_swz(r)) << 4) + 8 * (c & 1)) =
+            make_uint2(T::pack2(v[0], v[1]), T::pack2(v[2], v[3]));
+      } else {
+        *reinterpret_cast<uint4v*>(tile + r * G::RB + ((c ^ G::row_swz(r)) << 4)) = raw[i];
+      }
+    }
+  }
+  __device__ __forceinline__ typename T::vec8 operand(const char* tile, int s) const {
+    const int lane = lane_id();
+    return read_row_chunk<C, typename T::vec8>(tile, lane & 31, 2 * s + (lane >> 5));
+  }
+};
+
+// The same without the LDS tile, for the one kernel whose weights leave no room for it (three matrices of 128 rows):
+// every lane reads its own token's row and keeps it.
+template <typename T, bool IN32, int C>
+struct XStripLane {
+  static constexpr int KS = C / 16;
+  static constexpr int N = IN32 ? 2 * KS : KS;
+  static constexpr int kTileBytes = 0;
+  uint4v raw[N];
+  __device__ __forceinline__ void load(const void* x, int64_t batch_row0, int tok0, int last) {
+    const int lane = lane_id();
+    const int64_t elem0 = (batch_row0 + min(tok0 + (lane & 31), last)) * C + 8 * (lane >> 5);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       if (IN32)
@@ -75,8 +127,8 @@ struct XStrip {
         raw[i] = *reinterpret_cast<const uint4v*>(static_cast<const uint16_t*>(x) + elem0 + 16 * i);
     }
   }
-  template <typename T>
-  __device__ __forceinline__ typename T::vec8 operand(int s) const {
+  __device__ __forceinline__ void to_lds(char*) const {}
+  __device__ __forceinline__ typename T::vec8 operand(const char*, int s) const {
     if constexpr (IN32) {
       const float4v lo = __builtin_bit_cast(float4v, raw[2 * s]), hi = __builtin_bit_cast(float4v, raw[2 * s + 1]);
       const uint4v v = {T::pack2(lo[0], lo[1]), T::pack2(lo[2], lo[3]), T::pack2(hi[0], hi[1]), T::pack2(hi[2], hi[3])};
@@ -148,9 +200,11 @@ __global__ void __launch_bounds__(kSbThreads) linblk_kv_kernel(const SmallBlockP
   typedef typename T::vec8 vec8;
   constexpr int C = 32 * H, KS = C / 16, WS = 2 * C + 16;
   constexpr int NW = NQ ? 3 : 2;  // matrices staged: [Wq,] Wk, Wv (rows of w_qkv in that order)
+  typedef typename std::conditional<NQ && H == 4, XStripLane<T, IN32, C>, XStrip<T, IN32, C>>::type XS;
   constexpr int kFoldBytes = kSbWaves * H * 16 * 64 * 4;
-  constexpr int kWBytes = NW * C * WS;
-  __shared__ __align__(16) char s_w[kWBytes > kFoldBytes ? kWBytes : kFoldBytes];
+  constexpr int kWBytes = NW * C * WS, kXBytes = kSbWaves * XS::kTileBytes;
+  // weights, then the waves' x tiles; the fold at the end reuses all of it
+  __shared__ __align__(16) char s_w[kWBytes + kXBytes > kFoldBytes ? kWBytes + kXBytes : kFoldBytes];
   __shared__ float s_b[NW * C];
   __shared__ float s_stat[kSbWaves][H][3][32];
 
@@ -163,11 +217,9 @@ __global__ void __launch_bounds__(kSbThreads) linblk_kv_kernel(const SmallBlockP
   const int nstrips = (p.S + kSbStrip - 1) / kSbStrip;
   const int strip_end = min(nstrips, (ch + 1) * p.strips_per_chunk);
   int strip = ch * p.strips_per_chunk + wave;
-  auto strip_elem0 = [&](int st) {  // rows past the end re-read the last one (masked where it matters)
-    return ((int64_t)b * p.S + min(min(st, nstrips - 1) * kSbStrip + n, p.S - 1)) * C + 8 * g;
-  };
-  XStrip<IN32, KS> xs;
-  xs.load(p.x, strip_elem0(strip));
+  XS xs;
+  char* xtile = s_w + kWBytes + wave * XS::kTileBytes;
+  xs.load(p.x, (int64_t)b * p.S, min(strip, nstrips - 1) * kSbStrip, p.S - 1);
 
   stage_rows<T, IN32, C, WS, false>(s_w, p.w_qkv, NQ ? 0 : C, NW * C);
   stage_bias<T, IN32>(s_b, p.b_qkv, NQ ? 0 : C, NW * C);
@@ -193,9 +245,14 @@ __global__ void __launch_bounds__(kSbThreads) linblk_kv_kernel(const SmallBlockP
   for (; strip < strip_end; strip += kSbWaves) {
     const int t0 = strip * kSbStrip;
     vec8 xa[KS];
+    xs.to_lds(xtile);
+    wave_lds_order();
 #pragma unroll
-    for (int s = 0; s < KS; ++s) xa[s] = xs.template operand<T>(s);
-    xs.load(p.x, strip_elem0(strip + kSbWaves));  // the next strip (past the wave's share: any valid rows, unused)
+    for (int s = 0; s < KS; ++s) xa[s] = xs.operand(xtile, s);
+    wave_lds_order();
+    // the next strip (past the wave's share: any valid rows, unused); fp32 rows take twice the registers while they
+    // are in flight and are requested after the strip's work instead, where fewer are live
+    if (!IN32) xs.load(p.x, (int64_t)b * p.S, min(strip + kSbWaves, nstrips - 1) * kSbStrip, p.S - 1);
     bool dead[16];  // token of register r lies past the end
 #pragma unroll
     for (int r = 0; r < 16; ++r) dead[r] = t0 + 8 * (r >> 2) + 4 * g + (r & 3) >= p.S;
@@ -269,6 +326,7 @@ __global__ void __launch_bounds__(kSbThreads) linblk_kv_kernel(const SmallBlockP
 #pragma unroll
       for (int s = 0; s < 2; ++s) acc[h] = T::mfma(as_operand<T>(vw, s), as_operand<T>(kw, s), acc[h]);
     }
+    if (IN32) xs.load(p.x, (int64_t)b * p.S, min(strip + kSbWaves, nstrips - 1) * kSbStrip, p.S - 1);
   }
 
   // ---- fold the waves (wave h merges head h), write the chunk's partial
@@ -330,8 +388,14 @@ template <typename T, bool IN32, int H, bool EA>
 __global__ void __launch_bounds__(kSbThreads) linblk_out_kernel(const SmallBlockParams p) {
   typedef typename T::vec8 vec8;
   constexpr int C = 32 * H, KS = C / 16, WS = 2 * C + 16;
+  typedef XStrip<T, IN32, C> XS;
+  constexpr int ES = IN32 ? 4 : 2;        // bytes per element of y
+  constexpr int YCH = 128 / ES;           // output channels per store round: 128 bytes of every token's row
+  constexpr int YROW = 144;               // row of the transposition buffer (bytes)
+  constexpr int kXTile = XS::kTileBytes > kSbStrip * YROW ? XS::kTileBytes : kSbStrip * YROW;  // the y rounds reuse the wave's x tile
   __shared__ __align__(16) char s_wq[C * WS];
   __shared__ __align__(16) char s_wo[C * WS];             // columns in operand slot order
+  __shared__ __align__(16) char s_x[kSbWaves * kXTile];
   __shared__ __align__(16) float s_bq[C];
   __shared__ __align__(16) float s_bo[C];
   __shared__ __align__(16) uint4v s_kv[H][2][2][64];      // [head][hi, lo][step][lane]: operand of O^T = KVn^T Qs^T
@@ -346,11 +410,9 @@ __global__ void __launch_bounds__(kSbThreads) linblk_out_kernel(const SmallBlock
   const int nstrips = (p.S + kSbStrip - 1) / kSbStrip;
   const int strip_end = min(nstrips, (ch + 1) * p.strips_per_chunk);
   int strip = ch * p.strips_per_chunk + wave;
-  auto strip_elem0 = [&](int st) {
-    return ((int64_t)b * p.S + min(min(st, nstrips - 1) * kSbStrip + n, p.S - 1)) * C + 8 * g;
-  };
-  XStrip<IN32, KS> xs;
-  xs.load(p.x, strip_elem0(strip));
+  XS xs;
+  char* xtile = s_x + wave * kXTile;
+  xs.load(p.x, (int64_t)b * p.S, min(strip, nstrips - 1) * kSbStrip, p.S - 1);
 
   stage_rows<T, IN32, C, WS, false>(s_wq, p.w_qkv, 0, C);
   stage_rows<T, IN32, C, WS, true>(s_wo, p.w_out, 0, C);
@@ -437,9 +499,12 @@ __global__ void __launch_bounds__(kSbThreads) linblk_out_kernel(const SmallBlock
     const int t0 = strip * kSbStrip;
     const int tok = t0 + n;
     vec8 xb[KS];
+    xs.to_lds(xtile);
+    wave_lds_order();
 #pragma unroll
-    for (int s = 0; s < KS; ++s) xb[s] = xs.template operand<T>(s);
-    xs.load(p.x, strip_elem0(strip + kSbWaves));
+    for (int s = 0; s < KS; ++s) xb[s] = xs.operand(xtile, s);
+    wave_lds_order();
+    xs.load(p.x, (int64_t)b * p.S, min(strip + kSbWaves, nstrips - 1) * kSbStrip, p.S - 1);
 
     vec8 of[H][2];  // O^T of head h as operand of the output projection
 #pragma unroll
@@ -499,7 +564,9 @@ __global__ void __launch_bounds__(kSbThreads) linblk_out_kernel(const SmallBlock
       of[h][1] = as_operand<T>(ow, 1);
     }
 
-    // y^T block cb: rows = output channels 32 cb + [0..32), column = this lane's token
+    // y^T block cb: rows = output channels 32 cb + [0..32), column = this lane's token.  The blocks of 128 bytes of
+    // every token's row are turned round in the wave's LDS tile (x is in registers by now) and leave as 16-byte
+    // pieces of whole 128-byte row segments, 8 rows per store instruction.
 #pragma unroll
     for (int cb = 0; cb < H; ++cb) {
       float16v yacc;
@@ -512,20 +579,30 @@ __global__ void __launch_bounds__(kSbThreads) linblk_out_kernel(const SmallBlock
 #pragma unroll
         for (int s = 0; s < 2; ++s)
           yacc = T::mfma(*reinterpret_cast<const vec8*>(s_wo + orow + 64 * h + 32 * s), of[h][s], yacc);
-      if (tok < p.S) {
+      const int cin = (32 * cb) % YCH;  // first channel of the block inside its round
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float4v b4 = *reinterpret_cast<const float4v*>(s_bo + 32 * cb + 8 * q + 4 * g);
-          const int64_t at = ((int64_t)b * p.S + tok) * C + 32 * cb + 8 * q + 4 * g;
-          if constexpr (IN32) {
-            const float4v v = {yacc[4 * q] + b4[0], yacc[4 * q + 1] + b4[1], yacc[4 * q + 2] + b4[2], yacc[4 * q + 3] + b4[3]};
-            *reinterpret_cast<float4v*>(static_cast<float*>(p.y) + at) = v;
-          } else {
-            const uint2 v = make_uint2(T::pack2(yacc[4 * q] + b4[0], yacc[4 * q + 1] + b4[1]),
-                                       T::pack2(yacc[4 * q + 2] + b4[2], yacc[4 * q + 3] + b4[3]));
-            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + at) = v;
-          }
+      for (int q = 0; q < 4; ++q) {
+        const float4v b4 = *reinterpret_cast<const float4v*>(s_bo + 32 * cb + 8 * q + 4 * g);
+        char* at = xtile + n * YROW + (cin + 8 * q + 4 * g) * ES;
+        if constexpr (IN32) {
+          const float4v v = {yacc[4 * q] + b4[0], yacc[4 * q + 1] + b4[1], yacc[4 * q + 2] + b4[2], yacc[4 * q + 3] + b4[3]};
+          *reinterpret_cast<float4v*>(at) = v;
+        } else {
+          *reinterpret_cast<uint2*>(at) = make_uint2(T::pack2(yacc[4 * q] + b4[0], yacc[4 * q + 1] + b4[1]),
+                                                    T::pack2(yacc[4 * q + 2] + b4[2], yacc[4 * q + 3] + b4[3]));
         }
+      }
+      if ((32 * cb + 32) % YCH == 0) {  // a round is complete
+        const int c0 = 32 * cb + 32 - YCH;  // its first channel
+        wave_lds_order();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 8 * i + (lane >> 3);
+          const uint4v v = *reinterpret_cast<const uint4v*>(xtile + r * YROW + 16 * (lane & 7));
+          if (t0 + r < p.S)
+            *reinterpret_cast<uint4v*>(static_cast<char*>(p.y) + (((int64_t)b * p.S + t0 + r) * C + c0) * ES + 16 * (lane & 7)) = v;
+        }
+        wave_lds_order();
       }
     }
   }
