@@ -196,6 +196,9 @@ BlockLayout block_layout(const FtLinBlockArgs& b, int kind, char* base) {
   l.a = a;
   l.lt = l.lin + align256(ft_workspace_bytes(kind, &a));
   l.total = l.lt + kLtWorkspace;
+  // the two-launch form of narrow models keeps its per-chunk partial matrices there instead (0 where it does not apply)
+  const size_t small = ft::small_block_workspace_bytes(b);
+  if (small > l.total) l.total = small;
   return l;
 }
 
