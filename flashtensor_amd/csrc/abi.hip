@@ -512,8 +512,8 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
 int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx, void* stream) {
   if (!score || !idx) return fail(FT_EINVAL, "score / idx pointer is null");
   if (rows < 1 || S < 1 || k < 1 || k > S) return fail(FT_EINVAL, "bad top-k shape rows=%lld S=%d k=%d", (long long)rows, S, k);
-  if (S > 8192 && k > 8192)
-    return fail(FT_EUNSUPPORTED, "top-k of rows longer than 8192 takes k <= 8192 (S=%d k=%d)", S, k);
+  if (S > 8192 && k > 16384)
+    return fail(FT_EUNSUPPORTED, "top-k of rows longer than 8192 takes k <= 16384 (S=%d k=%d)", S, k);
   if (rows > 0x7fffffffLL) return fail(FT_EUNSUPPORTED, "too many rows");
   hipError_t e = ft::launch_topk(score, rows, S, k, idx, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "topk launch");

@@ -173,7 +173,7 @@ int ft_linattn_block_fwd(const FtLinBlockArgs* b, int kind, int normalize_q, voi
 /* Heavy hitters: indices of the k largest entries of each row of score [rows, S] fp32, in descending
  * score order (ties: lower index first), written as int64 [rows, k].  Not in the reference, whose H2O
  * case ends at the score (cases/kernels/h2o.py:34-38).  Rows of up to 8192 entries are sorted whole (any k <= S); longer rows take
- * k <= 8192 (a radix select of the k-th score, then a sort of the k winners), FT_EUNSUPPORTED beyond. */
+ * k <= 16384 (a radix select of the k-th score, then a sort of the k winners), FT_EUNSUPPORTED beyond. */
 int ft_topk(const float* score, int64_t rows, int32_t S, int32_t k, int64_t* idx, void* stream);
 
 /* The tensor E[B,H,Sq,Skv] = -ln(u) drawn by the seeded KeyFormer mode, written to device memory

@@ -145,7 +145,7 @@ def test_linattn_and_topk_argument_checks(lib):
   assert lib.ft_linattn_fwd(ctypes.byref(h4), _lib.FT_OP_EA, 1, _lib.FT_F16, 0x5000, need, None) == _lib.FT_EINVAL
   assert lib.ft_topk(None, 1, 8, 2, 0x1000, None) == _lib.FT_EINVAL
   assert lib.ft_topk(0x1000, 1, 8, 9, 0x2000, None) == _lib.FT_EINVAL
-  assert lib.ft_topk(0x1000, 1, 16384, 8193, 0x2000, None) == _lib.FT_EUNSUPPORTED   # long rows: k <= 8192
+  assert lib.ft_topk(0x1000, 1, 32768, 16385, 0x2000, None) == _lib.FT_EUNSUPPORTED   # long rows: k <= 16384
 
 
 def test_linear_block_argument_checks(lib):
@@ -317,8 +317,8 @@ def test_ffi_module_workspace_and_validation_of_the_other_entry_points(ffi):
     ffi.avgpool1d(0x1000, 4, 64, 4, 0x2000)
   with pytest.raises(ValueError, match="top-k"):
     ffi.topk(0x1000, 4, 64, 65, 0x2000)
-  with pytest.raises(RuntimeError, match="8192"):
-    ffi.topk(0x1000, 4, 8200, 8193, 0x2000)
+  with pytest.raises(RuntimeError, match="16384"):
+    ffi.topk(0x1000, 4, 20000, 16385, 0x2000)
   with pytest.raises(ValueError, match="kind"):
     ffi.linattn_fwd(a, ffi.OP_ATTN, 1, ffi.F16, 0x6000, 1 << 20)
   with pytest.raises(ValueError, match="3 entries"):

@@ -397,7 +397,7 @@ def test_topk_matches_torch_and_orders_ties(gpu):
     for k in sorted({1, max(1, S // 8), S}):
       assert torch.equal(ops.topk(x, k), torch.topk(x, k).indices), (S, k)
   # rows longer than the whole-row sort holds: select + sort of the winners
-  for S, ks in ((8193, (1, 1024, 8192)), (16384, (2048, 8191)), (40000, (5000,)), (131072, (1, 16384 // 2))):
+  for S, ks in ((8193, (1, 1024, 8192)), (16384, (2048, 8191)), (40000, (5000,)), (131072, (1, 8192, 16384))):
     x = torch.randn(3, S, generator=g).to(gpu)
     for k in ks:
       assert torch.equal(ops.topk(x, k), torch.topk(x, k).indices), (S, k)
@@ -407,8 +407,9 @@ def test_topk_matches_torch_and_orders_ties(gpu):
   assert torch.equal(got, want)
   same = torch.full((1, 9000), 2.5, device=gpu)
   assert torch.equal(ops.topk(same, 8192), torch.arange(8192, device=gpu)[None])
-  with pytest.raises(RuntimeError, match="8192"):
-    ops.topk(torch.zeros(1, 9000, device=gpu), 8193)
+  assert torch.equal(ops.topk(same.expand(2, 9000).contiguous(), 9000)[1], torch.arange(9000, device=gpu))   # k == S > 8192
+  with pytest.raises(RuntimeError, match="16384"):
+    ops.topk(torch.zeros(1, 20000, device=gpu), 16385)
   flat = torch.zeros(2, 700, device=gpu)
   assert torch.equal(ops.topk(flat, 700), torch.arange(700, device=gpu).expand(2, 700))
   spec = torch.tensor([[0.0, float("inf"), -float("inf"), 2.0, -0.0, 1e-40]], device=gpu)
