@@ -66,7 +66,14 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, CAUSA
   // pass, loses that balance here: measured 974 against 955 us for the B4 H32 S4096 sum-of-squares call, 267
   // against 239 us at B1.)
   const int bh = blockIdx.x % BH;
-  const int jb = blockIdx.x / BH;
+  int jb = blockIdx.x / BH;
+  if (p.pair_order) {
+    // Two workgroups per CU, all resident from the start: nothing is left to hand out as CUs free up, so the heavy half
+    // is dealt first, descending, and the light half after it ascending, which puts a heavy and a light block on the
+    // same CU (as in the attention pass).
+    const int nJB = gridDim.x / BH, half = (nJB + 1) / 2;
+    jb = jb < half ? jb : nJB - 1 - (jb - half);
+  }
   const int b = bh / p.H, h = bh % p.H;
   const int j0 = jb * BK;
   const int lane = lane_id(), wave = wave_id();
@@ -557,11 +564,16 @@ __global__ void __launch_bounds__(kColThreads, (colstats_waves_per_simd<T, CAUSA
 
 // ---------------------------------------------------------------------------------------------------
 
+int device_cu_count();  // attn_fwd.hip
+
 template <typename T, int D, bool CAUSAL, bool EMU, int MODE>
 static hipError_t launch_one(const ColstatsKernelParams& p, hipStream_t stream) {
   const int nJB = (p.Skv + kColBK - 1) / kColBK;
   dim3 grid((unsigned)(nJB * p.B * p.H));
-  hipLaunchKernelGGL((colstats_kernel<T, D, CAUSAL, EMU, MODE>), grid, dim3(kColThreads), 0, stream, p);
+  ColstatsKernelParams pp = p;
+  const int64_t cus = device_cu_count();
+  pp.pair_order = CAUSAL && (int64_t)grid.x > cus && (int64_t)grid.x <= 2 * cus;
+  hipLaunchKernelGGL((colstats_kernel<T, D, CAUSAL, EMU, MODE>), grid, dim3(kColThreads), 0, stream, pp);
   return hipGetLastError();
 }
 

@@ -52,6 +52,7 @@ struct ColstatsKernelParams {
   uint32_t pk_hi2, pk_lo2;  // as in AttnKernelParams
   float inv_tau;
   int group;  // query heads per k head
+  int pair_order;  // key-block order for launches of two workgroups per CU: heavy half descending, light half ascending (launcher)
 };
 
 // what happens to a logit between the scaled QK^T and the softmax of the attention pass
