@@ -696,12 +696,11 @@ __global__ void __launch_bounds__(64 * WAVES, (KF == kKfTensorLds ? 1 : 8 / WAVE
     wait_vmem();
     __syncthreads();
     if (kErLds && it < nw) {
-      // this tile's slice from LDS to registers, then the next tile's on its way into the same slots: in flight
-      // for the whole tile without holding a register.  The reads must have returned before the loads may
-      // overwrite their slots (nothing in the hardware orders an LDS read against a later direct-to-LDS load).
+      // this tile's slice from LDS to registers; the next tile's is requested into the same slots further down.  The
+      // reads must have returned before those loads may overwrite their slots (nothing in the hardware orders an LDS
+      // read against a later direct-to-LDS load).
       read_er(er);
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-      if (it + 1 < nw) issue_er(it + 1);
     }
     stage_k(it + 1, odd ? ldsK0 : ldsK1);
     stage_v(it + 1, odd ? ldsV0 : ldsV1);
@@ -716,6 +715,12 @@ __global__ void __launch_bounds__(64 * WAVES, (KF == kKfTensorLds ? 1 : 8 / WAVE
         else
           softmax_half(std::true_type{}, s, pb, it * BN + 32 * mbk, odd ? 1 : 0, mbk, er[mbk]);
         if (KF == kKfTensor && it + 1 < nw) load_er_half(er[mbk], it + 1, mbk);
+        // The next tile's noise, in flight for the rest of the tile without holding a register.  Requested here, behind
+        // the first half's contraction and softmax, rather than at the top of the tile in front of the K / V staging
+        // loads: the eight loads no longer queue up with the staging at the moment every wave leaves the barrier
+        // (B1 H32 S4096, same process: 538 -> 512 us per call; before the softmax 523, after the first half's PV 516,
+        // four loads behind each half's softmax 524).
+        if (kErLds && mbk == 0 && it + 1 < nw) issue_er(it + 1);
         pv_half(pb, odd ? ldsV1 : ldsV0, mbk);
       }
     }
