@@ -127,6 +127,13 @@ __device__ __forceinline__ float tanh_exp_form(float y) {
 
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
+// Orders one wave's LDS traffic for the compiler (a wave-private tile written by some lanes and read by others); the
+// hardware already executes a wave's LDS instructions in order.
+__device__ __forceinline__ void wave_lds_order() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
 // ---------------------------------------------------------------------------------------------------
 // A tile of ROWS x D 16-bit elements staged in LDS, rows of RB = 2 D bytes split in 16-byte chunks.
 // Two placements of chunk c of row r:

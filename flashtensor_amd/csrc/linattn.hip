@@ -107,13 +107,6 @@ size_t linattn_workspace_bytes(const FtAttnArgs& a0, int) {
   return (bytes + 255) & ~(size_t)255;
 }
 
-// Orders one wave's LDS traffic for the compiler; the hardware already executes a wave's LDS
-// instructions in order.
-__device__ __forceinline__ void wave_lds_order() {
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-}
-
 // One wave's private strip of ROWS tokens x 64 channels (128-byte rows): lane l moves the 16-byte chunk
 // l % 8 of rows l / 8 + 8 i, global -> registers -> LDS, so every load instruction covers 8 whole rows.
 // Rows past the end of the sequence re-read the last token (callers mask them).

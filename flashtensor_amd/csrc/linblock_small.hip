@@ -61,11 +61,6 @@ __device__ __forceinline__ uint4v load8(const void* base, int64_t elem) {
   }
 }
 
-__device__ __forceinline__ void wave_lds_order() {  // for the compiler; a wave's LDS instructions execute in order
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-}
-
 // A 32-token strip of x on its way to a wave: requested one strip ahead with loads that cover whole rows (lane l takes
 // a 16-byte chunk of row l / CPR + RPI i: an instruction touches 8 cache lines; with every lane reading its own
 // token's row it touched 32, and the address path showed), parked in the wave's LDS tile when the strip's turn comes
