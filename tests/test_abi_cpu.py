@@ -169,6 +169,10 @@ def test_linear_block_argument_checks(lib):
   assert lib.ft_linattn_block_fwd(ctypes.byref(odd), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
   f32 = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F32)
   assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(f32), _lib.FT_OP_EA) >= 2 * 100 * 4 * C * 4 + (32 << 20)
+  # narrow models in many short batches: the workspace also has to hold the two-launch form's partial matrices
+  # (1120 floats per batch, chunk and head), more here than the library form's q / k / v
+  many = _lib.FtLinBlockArgs(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 200000, 1, 4, 32, _lib.FT_F16)
+  assert lib.ft_linattn_block_workspace_bytes(ctypes.byref(many), _lib.FT_OP_SIMA) >= 200000 * 4 * 1120 * 4
   nul = _lib.FtLinBlockArgs(0x1000, None, 0x3000, 0x4000, 0x5000, 0x6000, 2, 100, 4, 64, _lib.FT_F16)
   assert lib.ft_linattn_block_fwd(ctypes.byref(nul), _lib.FT_OP_EA, 1, 0x10000, need, None) == _lib.FT_EINVAL
 
