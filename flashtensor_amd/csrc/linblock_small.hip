@@ -606,9 +606,9 @@ __global__ void __launch_bounds__(kSbThreads) linblk_out_kernel(const SmallBlock
 // ---------------------------------------------------------------------------------------------------
 int device_cu_count();  // attn_fwd.hip
 
-// Chunking of the token axis, or nch = 0 where this path does not apply: heads of 32 channels, 2 or 4 of them, and
-// enough batches that at most kSbMaxChunks chunks each occupy half of the CUs or more (every workgroup of pass 2
-// merges all chunks of its batch, holding one entry per chunk and matrix row in registers).
+// Chunking of the token axis, or nch = 0 where this path does not apply: heads of 32 channels, 2 or 4 of them, in at
+// most kSbMaxChunks chunks per batch (every workgroup of pass 2 merges all chunks of its batch, holding one entry per
+// chunk and matrix row in registers).
 void small_block_plan(const FtLinBlockArgs& a, int* nch, int* strips_per_chunk) {
   *nch = 0;
   *strips_per_chunk = 0;
@@ -618,7 +618,12 @@ void small_block_plan(const FtLinBlockArgs& a, int* nch, int* strips_per_chunk) 
   const int want = (int)std::min<int64_t>(std::min(nstrips, kSbMaxChunks), std::max<int64_t>(1, ((int64_t)cus + a.B - 1) / a.B));
   const int spc = (nstrips + want - 1) / want;
   const int n = (nstrips + spc - 1) / spc;
-  if ((int64_t)a.B * n * 2 < cus) return;  // too few workgroups for the chip: the library GEMMs do better
+  // Short calls are launch-bound and two launches beat the library form's five whatever the size (B1 S784: 21 against
+  // 33 us); with more than two strips per wave the workgroups must also cover a good part of the chip, or the
+  // library GEMMs, which spread any token count over all of it, do better (B4 S4096: 55 against 44 us; B16: 57
+  // against 68).
+  const int strips_per_wave = (spc + kSbWaves - 1) / kSbWaves;
+  if (strips_per_wave > 2 && (int64_t)a.B * n * 4 < cus) return;
   *nch = n;
   *strips_per_chunk = spc;
 }

@@ -147,7 +147,7 @@ int ft_linattn_fwd(const FtAttnArgs* a, int kind, int normalize_q, int out_dtype
  * bf16, or the .mlir's own fp32) and contiguous; biases may be NULL.  The two projections are hipBLASLt GEMMs (fp32
  * accumulation, bias added before the one rounding to the tensor type); q/k/v and the core's result live in the
  * workspace as tensors of that type.  D = 64, or 32 with an even H.
- * Narrow models (D = 32 with 2 or 4 heads, the .mlir's own geometry, and batches enough to fill the chip) run as
+ * Narrow models (D = 32 with 2 or 4 heads, the .mlir's own geometry; short calls, or batches enough to cover the chip) run as
  * two launches of this library's own instead: projection weights in LDS, q / k / v never leave registers, MFMA
  * operands of the tensor type (fp16 for fp32 tensors: x and the weights are rounded as they are loaded), no
  * hipBLASLt involved. */
