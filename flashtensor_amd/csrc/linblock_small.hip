@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(kSbThreads) linblk_kv_kernel(const SmallBlockP
   const int g = lane >> 5, n = lane & 31;
   const float NEG_INF = -__builtin_inff();
 
-  // the wave's strips: chunk's first + wave, + 4, ...; the first one is requested before anything else
+  // the wave's strips: chunk's first + wave, + kSbWaves, ...; the first one is requested before anything else
   const int nstrips = (p.S + kSbStrip - 1) / kSbStrip;
   const int strip_end = min(nstrips, (ch + 1) * p.strips_per_chunk);
   int strip = ch * p.strips_per_chunk + wave;
