@@ -609,13 +609,14 @@ __global__ void __launch_bounds__(kLinThreads) linattn_merge_kernel(const LinPar
     accv[i] *= s_scale[drow[i]];
     gmax = fmaxf(gmax, __builtin_fabsf(accv[i]));
   }
-  s_red[t] = gmax;
+  // the block's maximum: inside each wave by lane exchanges, then one value per wave through LDS
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o));
+  __syncthreads();  // every use of s_red above is over
+  if ((t & 63) == 0) s_red[t >> 6] = gmax;
   __syncthreads();
-  for (int s = kLinThreads / 2; s > 0; s >>= 1) {
-    if (t < s) s_red[t] = fmaxf(s_red[t], s_red[t + s]);
-    __syncthreads();
-  }
-  gmax = s_red[0];
+  gmax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+  static_assert(kLinThreads == 256, "four waves");
   // power-of-two scale that puts the largest entry of the block in [2^13, 2^14)
   int ex = 0;
   if (gmax > 0.f && gmax < __builtin_inff()) ex = 13 - (int)__builtin_floorf(__builtin_log2f(gmax));
