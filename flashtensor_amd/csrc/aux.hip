@@ -132,7 +132,8 @@ __global__ void __launch_bounds__(NT) topk_kernel(const float* __restrict__ scor
 //      entry before T, and of the entries equal to T the ones with the smallest indices (a workgroup-wide prefix count
 //      in index order), as the full sort would have ranked them;
 //   3. a bitonic network over those <= 16384 words in LDS, and the indices go out in rank order.
-// The same answers as the register sort, ties and NaNs (which sort first, as in torch.topk) included.
+// The same answers as the register sort, ties and NaNs included (a NaN of positive sign has the largest order key and
+// sorts first, as in torch.topk).
 constexpr int kTopkSelectMax = 16384;  // 128 KB of LDS for the winners: k = S / 8 up to S = 131072
 constexpr int kTopkSelectThreads = 1024;
 
